@@ -131,7 +131,7 @@ class ContinuousBatcher:
     def __init__(self, model, max_slots: int = 8, max_seq: int = None,
                  dtype=torch.float32, device=None,
                  prefill_chunk: int = 0, cache_cls=None,
-                 token_budget: int = 0):
+                 token_budget: int = 0, max_tokens: int = 0):
         """``prefill_chunk`` > 0 bounds prompt tokens prefetched per step
         (Dynamic SplitFuse: long prompts stream in across iterations so the
         decode batch's latency stays flat; reference inference/v2
@@ -142,16 +142,31 @@ class ContinuousBatcher:
         tokens — the whole decode batch plus up to the remaining budget of
         prefill-chunk tokens — so prefill never stalls decode and each
         step's work is a constant ~token_budget tokens (reference Dynamic
-        SplitFuse scheduling, inference/v2)."""
+        SplitFuse scheduling, inference/v2).
+
+        ``max_tokens`` sizes a model-provided paged cache: the most tokens
+        live at once, each request rounded up to whole blocks (default
+        ``max_slots * max_seq``)."""
         self.model = model
         cfg = model.cfg
         self.device = device or next(model.parameters()).device
         max_seq = max_seq or cfg.max_seq_len
-        kv_heads = getattr(cfg, "num_kv_heads", None) or cfg.num_heads
-        cache_cls = cache_cls or RaggedKVCache
-        self.cache = cache_cls(cfg.num_layers, max_slots, kv_heads,
-                               max_seq, cfg.head_dim, dtype=dtype,
-                               device=self.device)
+        # A model whose layers cache something other than per-head K/V
+        # brings its own manager (``build_cache``); such caches describe a
+        # step as a flat ragged batch instead of padded rows + mask.
+        self.ragged = hasattr(model, "build_cache")
+        if self.ragged:
+            self.cache = model.build_cache(
+                max_slots, max_tokens or max_slots * max_seq, dtype=dtype,
+                device=self.device)
+            if token_budget <= 0:
+                token_budget = 2048
+        else:
+            kv_heads = getattr(cfg, "num_kv_heads", None) or cfg.num_heads
+            cache_cls = cache_cls or RaggedKVCache
+            self.cache = cache_cls(cfg.num_layers, max_slots, kv_heads,
+                                   max_seq, cfg.head_dim, dtype=dtype,
+                                   device=self.device)
         self.free_slots = deque(range(max_slots))
         self.pending: deque = deque()
         self.active: Dict[int, Request] = {}
@@ -189,11 +204,104 @@ class ContinuousBatcher:
 
     def _admit(self):
         while self.pending and self.free_slots:
+            if self.ragged and not self._fits(self.pending[0]):
+                break        # wait for blocks; keeps arrival order
             req = self.pending.popleft()
-            req.slot = self.free_slots.popleft()
+            self._take_slot(req)
+
+    def _take_slot(self, req: Request):
+        req.slot = self.free_slots.popleft()
+        if self.ragged:
+            self.cache.reset_slot(req.slot)
+        else:
             self.cache.free(req.slot)
             self.cache.lens[req.slot] = 0
-            self.active[req.uid] = req
+        self.active[req.uid] = req
+
+    def _blocks_for(self, req: Request) -> int:
+        bs = self.cache.block_size
+        return (req.prompt.numel() + req.max_new_tokens + bs - 1) // bs
+
+    def _fits(self, req: Request) -> bool:
+        """Admission control for a paged pool: a request enters only if the
+        blocks it can grow to are not promised to the live ones."""
+        promised = sum(self._blocks_for(r) for r in self.active.values())
+        return promised + self._blocks_for(req) <= self.cache.num_blocks
+
+    # ------------------------------------------------ externally driven steps
+    def open(self, uid, max_new_tokens: int = 0) -> Request:
+        """Admit a request whose tokens the caller feeds step by step
+        (replaying a recorded schedule, speculative drivers, tests)."""
+        assert self.ragged, "open/feed/close need a ragged cache"
+        if not self.free_slots:
+            raise RuntimeError("no free request slot")
+        req = Request(uid=uid, prompt=torch.empty(0, dtype=torch.long),
+                      max_new_tokens=max_new_tokens)
+        self._take_slot(req)
+        return req
+
+    @torch.no_grad()
+    def feed(self, entries, rows=None):
+        """ONE model step over a ragged batch: ``entries`` is a list of
+        (request, tokens) — a prompt portion for some, one decoded token for
+        others. Returns logits for the flat token positions ``rows`` (default:
+        every token). This is the step the scheduler itself runs."""
+        slots = [r.slot for r, _ in entries]
+        counts = [len(t) for _, t in entries]
+        ids = torch.tensor([int(x) for _, t in entries for x in t],
+                           dtype=torch.long).to(self.device)
+        self.cache.begin_ragged(slots, counts)
+        try:
+            if rows is not None:
+                rows = torch.as_tensor(rows, dtype=torch.long).to(self.device)
+            logits = self.model(ids, kv_cache=self.cache, rows=rows)
+        finally:
+            self.cache.end_step()
+        return logits
+
+    def close(self, req: Request):
+        """Give a request's slot and blocks back."""
+        req.done = True
+        self.cache.free(req.slot)
+        self.free_slots.append(req.slot)
+        self.active.pop(req.uid, None)
+
+    @torch.no_grad()
+    def _step_ragged(self) -> List[Request]:
+        """Token-budgeted iteration on a ragged cache: every decoding request
+        contributes its last token, prompts fill the rest of the budget in
+        portions; one forward for all of it."""
+        self._admit()
+        finished = self._retire()
+        entries, budget = [], self.token_budget
+        for r in self.active.values():
+            if not r.in_prefill:
+                entries.append((r, [r.generated[-1]], 0))
+                budget -= 1
+        for r in self.active.values():
+            if r.in_prefill and budget > 0:
+                chunk = min(budget, r.prompt.numel() - r.prefilled)
+                if self.prefill_chunk > 0:
+                    chunk = min(chunk, self.prefill_chunk)
+                entries.append(
+                    (r, r.prompt[r.prefilled:r.prefilled + chunk].tolist(),
+                     chunk))
+                budget -= chunk
+        if not entries:
+            return finished
+        last, at, sampled = [], 0, []
+        for r, toks, chunk in entries:
+            at += len(toks)
+            if chunk == 0 or r.prefilled + chunk == r.prompt.numel():
+                last.append(at - 1)
+                sampled.append(r)
+        logits = self.feed([(r, t) for r, t, _ in entries], rows=last) \
+            if last else self.feed([(r, t) for r, t, _ in entries], rows=[0])
+        for r, _, chunk in entries:
+            r.prefilled += chunk
+        for i, r in enumerate(sampled):
+            r.generated.append(r.select(logits[i]))
+        return finished
 
     def _retire(self) -> List[Request]:
         finished = []
@@ -265,6 +373,8 @@ class ContinuousBatcher:
     @torch.no_grad()
     def step(self) -> List[Request]:
         """One scheduling iteration; returns requests finished this step."""
+        if self.ragged:
+            return self._step_ragged()
         if self.token_budget > 0:
             return self._step_packed()
         # 1) admit queued requests into free slots

@@ -10,6 +10,9 @@ from .falcon import (FalconConfig, FalconForCausalLM, falcon_7b,
                      falcon_mini, falcon_mini_gqa)
 from .mixtral import (MixtralConfig, MixtralForCausalLM, mixtral_8x7b,
                       mixtral_tiny, mixtral_mini)
+from .fizesun import FizesunConfig, FizesunForCausalLM, fizesun_tiny
+from .registry import (architectures, build_model, load_pretrained,
+                       register_architecture)
 
 __all__ = [
     "LlamaConfig", "LlamaForCausalLM", "llama3_8b", "llama3_1_8b", "llama3_70b",
@@ -20,4 +23,7 @@ __all__ = [
     "falcon_mini_gqa",
     "MixtralConfig", "MixtralForCausalLM",
     "mixtral_8x7b", "mixtral_tiny", "mixtral_mini",
+    "FizesunConfig", "FizesunForCausalLM", "fizesun_tiny",
+    "architectures", "build_model", "load_pretrained",
+    "register_architecture",
 ]

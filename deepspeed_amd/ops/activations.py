@@ -1,0 +1,38 @@
+"""Feed-forward activations used by the serving models (beside swiglu/geglu).
+
+* ``xielu(z, p, q)``: for z > 0 ``softplus(p) z^2 + z/2``; otherwise
+  ``(1/2 + softplus(q)) (exp(z) - 1 - z) + z/2``. p and q are learned
+  numbers of the layer.
+* ``clamped_swiglu(gu, limit)``: with ``g = min(gate, limit)`` and
+  ``u = clamp(up, -limit, limit)``: ``g * sigmoid(1.702 g) * (u + 1)``;
+  ``gu`` holds gate and up side by side ([T, 2F] -> [T, F]).
+Both evaluate in fp32 and round once.
+"""
+
+import torch
+import torch.nn.functional as F
+
+SWISH_SLOPE = 1.702
+
+
+def xielu(z, pq):
+    """z [T, F]; pq a 2-element fp32 tensor (p, q)."""
+    if z.is_cuda:
+        from . import serving_kernels as sk
+        return sk.xielu(z, pq)
+    zf = z.float()
+    a = F.softplus(pq[0].float())
+    b = 0.5 + F.softplus(pq[1].float())
+    neg = b * (torch.expm1(zf.clamp(max=0)) - zf) + 0.5 * zf
+    pos = a * zf * zf + 0.5 * zf
+    return torch.where(zf > 0, pos, neg).to(z.dtype)
+
+
+def clamped_swiglu(gu, limit):
+    if gu.is_cuda:
+        from . import serving_kernels as sk
+        return sk.clamped_swiglu(gu, limit)
+    f = gu.shape[-1] // 2
+    g = gu[..., :f].float().clamp(max=limit)
+    u = gu[..., f:].float().clamp(-limit, limit)
+    return (g * torch.sigmoid(SWISH_SLOPE * g) * (u + 1)).to(gu.dtype)

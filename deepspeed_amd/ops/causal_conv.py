@@ -1,0 +1,45 @@
+"""Short depthwise causal convolution over time with carried state, for
+ragged serving batches.
+
+``y_t = h_t + sum_j w[:, j] * h_(t - taps + 1 + j)`` per channel, with zeros
+before a sequence's start. A sequence's last ``taps - 1`` inputs are its
+carried state (``state[slot]``, oldest first), so a step that brings only a
+portion of a sequence continues exactly where the previous one stopped.
+
+The serving form fuses the preceding single-gain RMS norm: the kernel reads
+the fp32 residual stream, normalises in fp32, rounds the normed input ``h``
+to the compute dtype (that rounded value is also what the state keeps, so
+the result does not depend on where a sequence was cut), and convolves.
+"""
+
+import torch
+
+
+def _norm(x, gain, eps, dtype):
+    xf = x.float()
+    return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+            * gain.float().reshape(())).to(dtype)
+
+
+def norm_conv_ragged(x, gain, eps, conv_w, state, batch, out_dtype):
+    """x [T, C] fp32 residual; conv_w [C, taps]; state [slots, taps-1, C]
+    (updated in place); batch: RaggedBatch. Returns h + conv(h) as
+    [T, C] ``out_dtype``."""
+    if x.is_cuda:
+        from . import serving_kernels as sk
+        return sk.norm_conv_ragged(x, gain, eps, conv_w, state, batch,
+                                   out_dtype)
+    taps = conv_w.shape[1]
+    h = _norm(x, gain, eps, out_dtype)
+    out = torch.empty_like(h)
+    wf = conv_w.float()
+    at = 0
+    for slot, count in zip(batch.slots, batch.counts):
+        hist = torch.cat([state[slot], h[at:at + count]], 0).float()
+        win = hist.unfold(0, taps, 1)                 # [count, C, taps]
+        out[at:at + count] = (hist[taps - 1:] +
+                              (win * wf).sum(-1)).to(out_dtype)
+        if taps > 1:
+            state[slot] = hist[-(taps - 1):].to(state.dtype)
+        at += count
+    return out

@@ -135,3 +135,32 @@ class FusedLayerNorm(torch.nn.Module):
 
     def forward(self, x):
         return _LayerNormFn.apply(x, self.weight, self.bias, self.eps)
+
+
+def scalar_rms_norm(x, gain, eps=1e-6, out_dtype=None):
+    """RMS norm whose gain is ONE number for all coordinates:
+    ``x * rsqrt(mean(x^2) + eps) * gain``. Statistics and the product are
+    fp32 whatever ``x`` is; the result is rounded once to ``out_dtype``.
+    x [T, C] (fp32 residual stream or 16-bit), gain a 0-d/1-element fp32
+    tensor."""
+    out_dtype = out_dtype or x.dtype
+    if x.is_cuda:
+        from . import serving_kernels as sk
+        return sk.scalar_rms_norm(x, gain, eps, out_dtype)
+    xf = x.float()
+    y = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) \
+        * gain.float().reshape(())
+    return y.to(out_dtype)
+
+
+class ScalarRMSNorm(torch.nn.Module):
+    """RMSNorm with a single learned gain (kept fp32)."""
+
+    def __init__(self, eps=1e-6):
+        super().__init__()
+        self.gain = torch.nn.Parameter(torch.ones(1, dtype=torch.float32),
+                                       requires_grad=False)
+        self.eps = eps
+
+    def forward(self, x, out_dtype=None):
+        return scalar_rms_norm(x, self.gain, self.eps, out_dtype)

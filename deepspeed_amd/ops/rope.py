@@ -111,3 +111,23 @@ def apply_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
     """Apply RoPE to [B, S, H, D] (rotate-half pairing i <-> i+D/2)."""
     assert x.dim() == 4, "apply_rope expects [B, S, H, D]"
     return _RopeFn.apply(x, cos, sin, positions)
+
+
+def rope_interleaved_(x: torch.Tensor, positions: torch.Tensor,
+                      cos: torch.Tensor, sin: torch.Tensor,
+                      rot_dims: int) -> torch.Tensor:
+    """In-place rotary embedding with ADJACENT pairing (2i, 2i+1) on the first
+    ``rot_dims`` entries of the last axis; the rest pass unchanged.
+    x [T, ..., n]; positions [T] int; cos/sin [max_pos, rot_dims/2] fp32
+    tables (``rope_tables(rot_dims, ...)``). The rotation is done in fp32 and
+    rounded once to x's dtype."""
+    T = x.shape[0]
+    half = rot_dims // 2
+    shape = [T] + [1] * (x.dim() - 2) + [half]
+    c = cos[positions.long()].view(shape)
+    s = sin[positions.long()].view(shape)
+    xr = x[..., :rot_dims].float().reshape(*x.shape[:-1], half, 2)
+    u, v = xr[..., 0], xr[..., 1]
+    out = torch.stack([u * c - v * s, v * c + u * s], dim=-1)
+    x[..., :rot_dims] = out.reshape(*x.shape[:-1], rot_dims).to(x.dtype)
+    return x
