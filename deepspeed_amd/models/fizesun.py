@@ -295,7 +295,7 @@ class FizesunForCausalLM(nn.Module):
         ids = input_ids.reshape(-1)
         dt = self.dtype
         max_pos = cache.max_seq
-        x0 = self.embed_norm(self.embed[ids], out_dtype=torch.float32)
+        x0 = self.embed_norm(self.embed, out_dtype=torch.float32, index=ids)
         x = x0.clone()
         for stream, (i, t, enters) in enumerate(self.runs):
             if enters:
@@ -304,9 +304,8 @@ class FizesunForCausalLM(nn.Module):
             x = self.layers[i](x, cache, stream, dt, max_pos)
             if taps is not None:
                 taps.append(x.clone())
-        if rows is not None:
-            x = x[rows]
-        return F.linear(self.final_norm(x, out_dtype=dt), self.head)
+        return F.linear(self.final_norm(x, out_dtype=dt, index=rows),
+                        self.head)
 
     def num_parameters(self):
         return sum(p.numel() for p in self.parameters())

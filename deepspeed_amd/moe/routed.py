@@ -16,8 +16,15 @@ import torch.nn.functional as F
 from ..ops.activations import clamped_swiglu
 
 
+def _sk():
+    from ..ops import serving_kernels
+    return serving_kernels
+
+
 def topk_softmax(logits, top):
     """logits [T, E] fp32 -> (idx [T, top] int64, weight [T, top] fp32)."""
+    if logits.is_cuda and _sk().enabled():
+        return _sk().topk_softmax(logits.float(), top)
     val, idx = torch.topk(logits.float(), top, dim=-1)
     return idx, torch.softmax(val, dim=-1)
 
@@ -27,8 +34,8 @@ def moe_combine(y, inv, weight, shared=None, shared_gate=None):
     sorted position of each (token, choice); weight [T, top] fp32. Returns
     sum_k weight[t, k] * y[inv[t, k]] (+ sigmoid(shared_gate[t]) *
     shared[t]) as [T, C] in y's dtype."""
-    if y.is_cuda:
-        from ..ops import serving_kernels as sk
+    if y.is_cuda and _sk().enabled():
+        sk = _sk()
         return sk.moe_combine(y, inv, weight, shared, shared_gate)
     out = (y.float()[inv] * weight[..., None]).sum(1)
     if shared is not None:

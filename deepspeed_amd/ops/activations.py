@@ -12,13 +12,18 @@ Both evaluate in fp32 and round once.
 import torch
 import torch.nn.functional as F
 
+def _sk():
+    from . import serving_kernels
+    return serving_kernels
+
+
 SWISH_SLOPE = 1.702
 
 
 def xielu(z, pq):
     """z [T, F]; pq a 2-element fp32 tensor (p, q)."""
-    if z.is_cuda:
-        from . import serving_kernels as sk
+    if z.is_cuda and _sk().enabled():
+        sk = _sk()
         return sk.xielu(z, pq)
     zf = z.float()
     a = F.softplus(pq[0].float())
@@ -29,8 +34,8 @@ def xielu(z, pq):
 
 
 def clamped_swiglu(gu, limit):
-    if gu.is_cuda:
-        from . import serving_kernels as sk
+    if gu.is_cuda and _sk().enabled():
+        sk = _sk()
         return sk.clamped_swiglu(gu, limit)
     f = gu.shape[-1] // 2
     g = gu[..., :f].float().clamp(max=limit)

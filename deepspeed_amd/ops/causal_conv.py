@@ -15,6 +15,11 @@ the result does not depend on where a sequence was cut), and convolves.
 import torch
 
 
+def _sk():
+    from . import serving_kernels
+    return serving_kernels
+
+
 def _norm(x, gain, eps, dtype):
     xf = x.float()
     return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
@@ -25,8 +30,8 @@ def norm_conv_ragged(x, gain, eps, conv_w, state, batch, out_dtype):
     """x [T, C] fp32 residual; conv_w [C, taps]; state [slots, taps-1, C]
     (updated in place); batch: RaggedBatch. Returns h + conv(h) as
     [T, C] ``out_dtype``."""
-    if x.is_cuda:
-        from . import serving_kernels as sk
+    if x.is_cuda and _sk().enabled():
+        sk = _sk()
         return sk.norm_conv_ragged(x, gain, eps, conv_w, state, batch,
                                    out_dtype)
     taps = conv_w.shape[1]

@@ -1,0 +1,612 @@
+// Ragged-batch serving kernels for MI355X (gfx950): single-gain RMS norm,
+// norm + short causal convolution with carried state, latent-attention
+// prologue/attention/epilogue over a paged row pool, feed-forward
+// activations and the routed-expert combine.
+//
+// Plain C ABI (raw device pointers + a hipStream_t) so the library builds in
+// seconds with hipcc alone and is loaded through ctypes. dtype codes:
+// 0 = float, 1 = bfloat16. Everything the models define as 32-bit (norm
+// statistics, rotations, scores, softmax, the weighted sums, router and
+// gates) is computed in float here whatever the storage type.
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_bf16.h>
+#include <stdint.h>
+
+namespace {
+
+using bf16 = __hip_bfloat16;
+
+__device__ __forceinline__ float ld(const float* p) { return *p; }
+__device__ __forceinline__ float ld(const bf16* p) { return __bfloat162float(*p); }
+__device__ __forceinline__ void st(float* p, float v) { *p = v; }
+__device__ __forceinline__ void st(bf16* p, float v) { *p = __float2bfloat16(v); }
+// value after one rounding to the storage type
+template <typename T> __device__ __forceinline__ float rnd(float v);
+template <> __device__ __forceinline__ float rnd<float>(float v) { return v; }
+template <> __device__ __forceinline__ float rnd<bf16>(float v) {
+  return __bfloat162float(__float2bfloat16(v));
+}
+
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o, 64);
+  return x;
+}
+__device__ __forceinline__ float wave_max(float x) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) x = fmaxf(x, __shfl_xor(x, o, 64));
+  return x;
+}
+
+constexpr int NT = 256;  // threads per block for the row kernels
+
+// every thread gets the block total; scratch holds NT/64 floats
+__device__ __forceinline__ float block_sum(float x, float* scratch) {
+  x = wave_sum(x);
+  if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = x;
+  __syncthreads();
+  float t = 0.f;
+  for (int i = 0; i < (int)(blockDim.x >> 6); ++i) t += scratch[i];
+  __syncthreads();
+  return t;
+}
+
+// ---------------------------------------------------------------- norm
+// out[r] = x[idx ? idx[r] : r] * rsqrt(mean(x^2) + eps) * gain
+template <typename TI, typename TO>
+__global__ __launch_bounds__(NT) void scalar_rms_norm_k(
+    const TI* __restrict__ x, const int64_t* __restrict__ idx,
+    const float* __restrict__ gain, TO* __restrict__ out, int C, float eps) {
+  __shared__ float red[NT / 64];
+  const int64_t r = blockIdx.x;
+  const TI* row = x + (idx ? idx[r] : r) * (int64_t)C;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < C; c += NT) {
+    float v = ld(row + c);
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  const float k = rsqrtf(ss / (float)C + eps) * gain[0];
+  for (int c = threadIdx.x; c < C; c += NT) st(out + r * C + c, ld(row + c) * k);
+}
+
+// ------------------------------------------------- norm + causal conv
+constexpr int MAXTAPS = 16;
+
+// One block per token. h = round_T(norm(x)); out = h_t + sum_k w[c][taps-1-k]
+// * h_(t-k). Earlier inputs come from this step's rows when the sequence
+// brought them, from the slot's tail otherwise, and are zero before position 0.
+template <typename T>
+__global__ __launch_bounds__(NT) void norm_conv_k(
+    const float* __restrict__ x, const float* __restrict__ gain,
+    const T* __restrict__ w, const T* __restrict__ state,
+    int64_t state_slot_stride, const int* __restrict__ cu,
+    const int* __restrict__ seq_slot, const int* __restrict__ tok_seq,
+    const int* __restrict__ tok_pos, T* __restrict__ out, int C, int taps,
+    float eps) {
+  __shared__ float red[NT / 64];
+  const int t = blockIdx.x;
+  const int s = tok_seq[t];
+  const int j = t - cu[s];
+  const int pos = tok_pos[t];
+  const int tail = taps - 1;
+  const T* sl = state + (int64_t)seq_slot[s] * state_slot_stride;
+  float scale[MAXTAPS];  // per distance k: norm factor of an in-step row
+  const float g = gain[0];
+  for (int k = 0; k < taps; ++k) {
+    scale[k] = 0.f;
+    if (k <= j) {  // block-uniform
+      const float* row = x + (int64_t)(t - k) * C;
+      float ss = 0.f;
+      for (int c = threadIdx.x; c < C; c += NT) ss += row[c] * row[c];
+      ss = block_sum(ss, red);
+      scale[k] = rsqrtf(ss / (float)C + eps) * g;
+    }
+  }
+  for (int c = threadIdx.x; c < C; c += NT) {
+    float h0 = rnd<T>(x[(int64_t)t * C + c] * scale[0]);
+    float acc = ld(w + (int64_t)c * taps + tail) * h0;
+    for (int k = 1; k < taps; ++k) {
+      float hk;
+      if (pos - k < 0) break;
+      if (k <= j)
+        hk = rnd<T>(x[(int64_t)(t - k) * C + c] * scale[k]);
+      else
+        hk = ld(sl + (int64_t)(tail + j - k) * C + c);
+      acc += ld(w + (int64_t)c * taps + tail - k) * hk;
+    }
+    st(out + (int64_t)t * C + c, h0 + acc);
+  }
+}
+
+// One block per sequence: the tail becomes the last taps-1 normed inputs.
+template <typename T>
+__global__ __launch_bounds__(NT) void conv_tail_k(
+    const float* __restrict__ x, const float* __restrict__ gain,
+    T* __restrict__ state, int64_t state_slot_stride,
+    const int* __restrict__ cu, const int* __restrict__ seq_slot,
+    const int* __restrict__ seq_start, int C, int taps, float eps) {
+  __shared__ float red[NT / 64];
+  const int s = blockIdx.x;
+  const int tail = taps - 1;
+  const int start = seq_start[s];
+  const int count = cu[s + 1] - cu[s];
+  T* sl = state + (int64_t)seq_slot[s] * state_slot_stride;
+  float scale[MAXTAPS];
+  const float g = gain[0];
+  for (int i = 0; i < tail; ++i) {
+    scale[i] = 0.f;
+    const int p = start + count - tail + i;  // absolute position kept at i
+    if (p >= start) {
+      const float* row = x + (int64_t)(cu[s] + p - start) * C;
+      float ss = 0.f;
+      for (int c = threadIdx.x; c < C; c += NT) ss += row[c] * row[c];
+      ss = block_sum(ss, red);
+      scale[i] = rsqrtf(ss / (float)C + eps) * g;
+    }
+  }
+  for (int c = threadIdx.x; c < C; c += NT) {
+    float v[MAXTAPS];
+    for (int i = 0; i < tail; ++i) {
+      const int p = start + count - tail + i;
+      if (p < 0)
+        v[i] = 0.f;
+      else if (p >= start)
+        v[i] = x[(int64_t)(cu[s] + p - start) * C + c] * scale[i];
+      else
+        v[i] = ld(sl + (int64_t)(i + count) * C + c);
+    }
+    for (int i = 0; i < tail; ++i) st(sl + (int64_t)i * C + c, v[i]);
+  }
+}
+
+// ------------------------------------------------------ latent prologue
+// proj row = [ q (H x (dim+rot)) | latent (rank) | k_rot (rot) | gate (H) ].
+template <typename T>
+__global__ __launch_bounds__(NT) void latent_prep_k(
+    const T* __restrict__ proj, int ld_proj, const float* __restrict__ norm_w,
+    const int* __restrict__ tok_pos, const int* __restrict__ tok_row,
+    const float* __restrict__ cosT, const float* __restrict__ sinT,
+    T* __restrict__ pool, T* __restrict__ q_nope, T* __restrict__ q_rot,
+    float* __restrict__ gate, int Ttok, int H, int dim, int rot, int rank,
+    int rot_dims, float eps) {
+  __shared__ float red[NT / 64];
+  const int t = blockIdx.x;
+  const T* p = proj + (int64_t)t * ld_proj;
+  const int nq = H * (dim + rot);
+  const int half = rot_dims >> 1;
+  const float* cs = cosT + (int64_t)tok_pos[t] * half;
+  const float* sn = sinT + (int64_t)tok_pos[t] * half;
+  T* row = pool + (int64_t)tok_row[t] * (rank + rot);
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < rank; c += NT) {
+    float v = ld(p + nq + c);
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  const float k = rsqrtf(ss / (float)rank + eps);
+  for (int c = threadIdx.x; c < rank; c += NT)
+    st(row + c, ld(p + nq + c) * k * norm_w[c]);
+  // shared rotated key part
+  for (int c = threadIdx.x; c < rot; c += NT) {
+    float v = ld(p + nq + rank + c);
+    if (c < rot_dims) {
+      const float o = ld(p + nq + rank + (c ^ 1));
+      const float co = cs[c >> 1], si = sn[c >> 1];
+      v = (c & 1) ? v * co + o * si : v * co - o * si;
+    }
+    st(row + rank + c, v);
+  }
+  // queries: rotated part [T, H, rot]; unrotated part regrouped [H, T, dim]
+  for (int i = threadIdx.x; i < H * rot; i += NT) {
+    const int h = i / rot, c = i - h * rot;
+    const T* q = p + h * (dim + rot) + dim;
+    float v = ld(q + c);
+    if (c < rot_dims) {
+      const float o = ld(q + (c ^ 1));
+      const float co = cs[c >> 1], si = sn[c >> 1];
+      v = (c & 1) ? v * co + o * si : v * co - o * si;
+    }
+    st(q_rot + ((int64_t)t * H + h) * rot + c, v);
+  }
+  for (int i = threadIdx.x; i < H * dim; i += NT) {
+    const int h = i / dim, c = i - h * dim;
+    q_nope[((int64_t)h * Ttok + t) * dim + c] = p[h * (dim + rot) + c];
+  }
+  for (int h = threadIdx.x; h < H; h += NT)
+    gate[(int64_t)t * H + h] = 1.f / (1.f + expf(-ld(p + nq + rank + rot + h)));
+}
+
+// ------------------------------------------------------ latent attention
+// Generic exact kernel: one block per (token, key split), heads in groups of
+// HG. Keys are staged through LDS in chunks (odd row stride: conflict-free
+// column reads); scores, online softmax and the weighted sum of latents are
+// float. With nsplit > 1 the block writes (max, sum, unnormalised sum) and
+// latent_attn_merge_k finishes.
+constexpr int HG = 8;
+constexpr int RPT = 4;  // latent columns per thread: rank <= RPT * NT
+
+template <typename T>
+__global__ __launch_bounds__(NT) void latent_attn_k(
+    const T* __restrict__ q_lat,  // [H, Ttok, rank]
+    const T* __restrict__ q_rot,  // [Ttok, H, rot]
+    const T* __restrict__ pool,   // rows of rank+rot
+    const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
+    const int* __restrict__ table, int maxb, int bs,
+    T* __restrict__ out,          // [H, Ttok, rank]
+    float* __restrict__ part,     // [Ttok, nsplit, H, rank + 2] when nsplit > 1
+    int Ttok, int H, int rank, int rot, int KC, int nsplit, float scale) {
+  extern __shared__ float smem[];
+  const int D = rank + rot;
+  const int DS = D | 1;
+  float* qs = smem;                       // [HG][D]
+  float* sc = qs + HG * D;                // [HG][KC]
+  float* alpha = sc + HG * KC;            // [HG] rescale of this chunk
+  float* mrun = alpha + HG;               // [HG] running max
+  float* lrun = mrun + HG;                // [HG] running sum
+  T* ks = reinterpret_cast<T*>(lrun + HG);   // [KC][DS]
+  const int t = blockIdx.x, split = blockIdx.y;
+  const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
+  const int s = tok_seq[t];
+  const int nkeys = tok_pos[t] + 1;
+  const int* tab = table + (int64_t)s * maxb;
+  // key range of this split, in whole chunks
+  const int nchunk = (nkeys + KC - 1) / KC;
+  const int cps = (nchunk + nsplit - 1) / nsplit;
+  const int c_lo = split * cps, c_hi = min(nchunk, c_lo + cps);
+
+  for (int h0 = 0; h0 < H; h0 += HG) {
+    const int nh = min(HG, H - h0);
+    __syncthreads();
+    for (int i = tid; i < nh * D; i += NT) {
+      const int h = i / D, c = i - h * D;
+      qs[i] = c < rank ? ld(q_lat + ((int64_t)(h0 + h) * Ttok + t) * rank + c)
+                       : ld(q_rot + ((int64_t)t * H + h0 + h) * rot + c - rank);
+    }
+    if (tid < HG) {
+      mrun[tid] = -INFINITY;
+      lrun[tid] = 0.f;
+    }
+    float acc[HG][RPT];
+#pragma unroll
+    for (int h = 0; h < HG; ++h)
+#pragma unroll
+      for (int i = 0; i < RPT; ++i) acc[h][i] = 0.f;
+    for (int ch = c_lo; ch < c_hi; ++ch) {
+      const int k0 = ch * KC;
+      const int nk = min(KC, nkeys - k0);
+      __syncthreads();
+      for (int i = tid; i < nk * D; i += NT) {
+        const int kk = i / D, c = i - kk * D;
+        const int p = k0 + kk;
+        const int64_t r = (int64_t)tab[p / bs] * bs + p % bs;
+        ks[kk * DS + c] = pool[r * D + c];
+      }
+      __syncthreads();
+      for (int i = tid; i < nh * KC; i += NT) {
+        const int h = i / KC, kk = i - h * KC;
+        float d = -INFINITY;
+        if (kk < nk) {
+          d = 0.f;
+          const float* q = qs + h * D;
+          const T* kr = ks + kk * DS;
+          for (int c = 0; c < D; ++c) d += q[c] * ld(kr + c);
+          d *= scale;
+        }
+        sc[i] = d;
+      }
+      __syncthreads();
+      // online softmax: wave w owns heads w, w + 4, ...; scores become weights
+      for (int h = wid; h < nh; h += NT / 64) {
+        float mx = -INFINITY;
+        for (int kk = lane; kk < nk; kk += 64) mx = fmaxf(mx, sc[h * KC + kk]);
+        mx = wave_max(mx);
+        const float m_old = mrun[h];
+        const float m_new = fmaxf(m_old, mx);
+        float psum = 0.f;
+        for (int kk = lane; kk < nk; kk += 64) {
+          const float p = expf(sc[h * KC + kk] - m_new);
+          sc[h * KC + kk] = p;
+          psum += p;
+        }
+        psum = wave_sum(psum);
+        if (lane == 0) {
+          const float a = expf(m_old - m_new);  // 0 on the first chunk
+          alpha[h] = a;
+          mrun[h] = m_new;
+          lrun[h] = lrun[h] * a + psum;
+        }
+      }
+      __syncthreads();
+#pragma unroll
+      for (int h = 0; h < HG; ++h) {
+        if (h < nh) {
+          const float a = alpha[h];
+#pragma unroll
+          for (int i = 0; i < RPT; ++i) acc[h][i] *= a;
+        }
+      }
+      // weighted sum of latents: thread owns columns tid + i*NT
+      for (int kk = 0; kk < nk; ++kk) {
+        float c[RPT];
+#pragma unroll
+        for (int i = 0; i < RPT; ++i) {
+          const int col = tid + i * NT;
+          c[i] = col < rank ? ld(ks + kk * DS + col) : 0.f;
+        }
+#pragma unroll
+        for (int h = 0; h < HG; ++h) {
+          if (h < nh) {
+            const float p = sc[h * KC + kk];
+#pragma unroll
+            for (int i = 0; i < RPT; ++i) acc[h][i] += p * c[i];
+          }
+        }
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int h = 0; h < HG; ++h) {
+      if (h < nh) {
+        if (nsplit == 1) {
+          const float inv = 1.f / lrun[h];
+#pragma unroll
+          for (int i = 0; i < RPT; ++i) {
+            const int col = tid + i * NT;
+            if (col < rank)
+              st(out + ((int64_t)(h0 + h) * Ttok + t) * rank + col, acc[h][i] * inv);
+          }
+        } else {
+          float* pp = part + (((int64_t)t * nsplit + split) * H + h0 + h) * (rank + 2);
+          if (tid == 0) {
+            pp[0] = mrun[h];
+            pp[1] = lrun[h];
+          }
+#pragma unroll
+          for (int i = 0; i < RPT; ++i) {
+            const int col = tid + i * NT;
+            if (col < rank) pp[2 + col] = acc[h][i];
+          }
+        }
+      }
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(NT) void latent_attn_merge_k(
+    const float* __restrict__ part, T* __restrict__ out, int Ttok, int H,
+    int rank, int nsplit) {
+  const int t = blockIdx.x, h = blockIdx.y;
+  float m = -INFINITY;
+  for (int s = 0; s < nsplit; ++s)
+    m = fmaxf(m, part[(((int64_t)t * nsplit + s) * H + h) * (rank + 2)]);
+  float l = 0.f;
+  for (int s = 0; s < nsplit; ++s) {
+    const float* pp = part + (((int64_t)t * nsplit + s) * H + h) * (rank + 2);
+    if (pp[1] > 0.f) l += pp[1] * expf(pp[0] - m);
+  }
+  for (int c = threadIdx.x; c < rank; c += NT) {
+    float a = 0.f;
+    for (int s = 0; s < nsplit; ++s) {
+      const float* pp = part + (((int64_t)t * nsplit + s) * H + h) * (rank + 2);
+      if (pp[1] > 0.f) a += pp[2 + c] * expf(pp[0] - m);
+    }
+    st(out + ((int64_t)h * Ttok + t) * rank + c, a / l);
+  }
+}
+
+// out[t, h*v + c] = o[h, t, c] * gate[t, h]
+template <typename T>
+__global__ void gate_merge_k(const T* __restrict__ o, const float* __restrict__ gate,
+                             T* __restrict__ out, int Ttok, int H, int v) {
+  const int64_t n = (int64_t)Ttok * H * v;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int c = i % v;
+    const int h = (i / v) % H;
+    const int64_t t = i / ((int64_t)v * H);
+    st(out + i, ld(o + ((int64_t)h * Ttok + t) * v + c) * gate[t * H + h]);
+  }
+}
+
+// ---------------------------------------------------------- activations
+__device__ __forceinline__ float softplusf(float x) {
+  return x > 20.f ? x : log1pf(expf(x));
+}
+
+template <typename T>
+__global__ void xielu_k(const T* __restrict__ z, const float* __restrict__ pq,
+                        T* __restrict__ out, int64_t n) {
+  const float a = softplusf(pq[0]);
+  const float b = 0.5f + softplusf(pq[1]);
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const float v = ld(z + i);
+    const float r = v > 0.f ? a * v * v + 0.5f * v : b * (expm1f(v) - v) + 0.5f * v;
+    st(out + i, r);
+  }
+}
+
+// gu [rows, 2F] (gate | up) -> out [rows, F]
+template <typename T>
+__global__ void clamped_swiglu_k(const T* __restrict__ gu, T* __restrict__ out,
+                                 int64_t rows, int F, float limit) {
+  const int64_t n = rows * F;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = i / F;
+    const int c = i - r * F;
+    const float g = fminf(ld(gu + r * 2 * F + c), limit);
+    const float u = fminf(fmaxf(ld(gu + r * 2 * F + F + c), -limit), limit);
+    st(out + i, g / (1.f + expf(-1.702f * g)) * (u + 1.f));
+  }
+}
+
+// out[t] = sum_k w[t,k] * y[inv[t,k]] (+ sigmoid(sg[t]) * shared[t])
+template <typename T>
+__global__ void moe_combine_k(const T* __restrict__ y, const int64_t* __restrict__ inv,
+                              const float* __restrict__ w, const T* __restrict__ shared,
+                              const T* __restrict__ sg, T* __restrict__ out,
+                              int top, int C) {
+  const int64_t t = blockIdx.x;
+  const float g = shared ? 1.f / (1.f + expf(-ld(sg + t))) : 0.f;
+  for (int c = threadIdx.x; c < C; c += blockDim.x) {
+    float a = 0.f;
+    for (int k = 0; k < top; ++k)
+      a += w[t * top + k] * ld(y + inv[t * top + k] * C + c);
+    if (shared) a += g * ld(shared + t * C + c);
+    st(out + t * C + c, a);
+  }
+}
+
+// per token: the `top` largest of E logits, softmax over them
+__global__ void topk_softmax_k(const float* __restrict__ z, int64_t* __restrict__ idx,
+                               float* __restrict__ w, int Ttok, int E, int top) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= Ttok) return;
+  const float* r = z + (int64_t)t * E;
+  float best = 0.f, sum = 0.f;
+  for (int k = 0; k < top; ++k) {
+    int bi = -1;
+    float bv = -INFINITY;
+    for (int e = 0; e < E; ++e) {
+      bool taken = false;
+      for (int q = 0; q < k; ++q) taken |= idx[(int64_t)t * top + q] == e;
+      if (!taken && (bi < 0 || r[e] > bv)) {
+        bi = e;
+        bv = r[e];
+      }
+    }
+    idx[(int64_t)t * top + k] = bi;
+    if (k == 0) best = bv;
+    const float p = expf(bv - best);
+    w[(int64_t)t * top + k] = p;
+    sum += p;
+  }
+  for (int k = 0; k < top; ++k) w[(int64_t)t * top + k] /= sum;
+}
+
+inline int nblocks(int64_t n, int b) {
+  int64_t g = (n + b - 1) / b;
+  return (int)(g < 1 ? 1 : (g > 4096 ? 4096 : g));
+}
+
+}  // namespace
+
+#define BY_DTYPE(dt, CALL)            \
+  do {                                \
+    if ((dt) == 0) {                  \
+      using T = float;                \
+      CALL;                           \
+    } else {                          \
+      using T = bf16;                 \
+      CALL;                           \
+    }                                 \
+  } while (0)
+
+extern "C" {
+
+int dsv_scalar_rms_norm(const void* x, int in_dt, const int64_t* idx, const float* gain,
+                        void* out, int out_dt, int rows, int C, float eps, hipStream_t s) {
+  if (rows <= 0) return 0;
+  if (in_dt == 0 && out_dt == 0)
+    scalar_rms_norm_k<float, float><<<rows, NT, 0, s>>>((const float*)x, idx, gain, (float*)out, C, eps);
+  else if (in_dt == 0)
+    scalar_rms_norm_k<float, bf16><<<rows, NT, 0, s>>>((const float*)x, idx, gain, (bf16*)out, C, eps);
+  else if (out_dt == 0)
+    scalar_rms_norm_k<bf16, float><<<rows, NT, 0, s>>>((const bf16*)x, idx, gain, (float*)out, C, eps);
+  else
+    scalar_rms_norm_k<bf16, bf16><<<rows, NT, 0, s>>>((const bf16*)x, idx, gain, (bf16*)out, C, eps);
+  return (int)hipGetLastError();
+}
+
+int dsv_norm_conv(const float* x, const float* gain, const void* w, void* state,
+                  int64_t state_slot_stride, const int* cu, const int* seq_slot,
+                  const int* seq_start, const int* tok_seq, const int* tok_pos, void* out,
+                  int dt, int Ttok, int nseq, int C, int taps, float eps, hipStream_t s) {
+  if (taps > MAXTAPS) return -1;
+  if (Ttok <= 0) return 0;
+  BY_DTYPE(dt, (norm_conv_k<T><<<Ttok, NT, 0, s>>>(x, gain, (const T*)w, (const T*)state,
+                                                    state_slot_stride, cu, seq_slot, tok_seq,
+                                                    tok_pos, (T*)out, C, taps, eps)));
+  if (taps > 1)
+    BY_DTYPE(dt, (conv_tail_k<T><<<nseq, NT, 0, s>>>(x, gain, (T*)state, state_slot_stride, cu,
+                                                      seq_slot, seq_start, C, taps, eps)));
+  return (int)hipGetLastError();
+}
+
+int dsv_latent_prep(const void* proj, int ld_proj, const float* norm_w, const int* tok_pos,
+                    const int* tok_row, const float* cosT, const float* sinT, void* pool,
+                    void* q_nope, void* q_rot, float* gate, int dt, int Ttok, int H, int dim,
+                    int rot, int rank, int rot_dims, float eps, hipStream_t s) {
+  if (Ttok <= 0) return 0;
+  BY_DTYPE(dt, (latent_prep_k<T><<<Ttok, NT, 0, s>>>(
+                   (const T*)proj, ld_proj, norm_w, tok_pos, tok_row, cosT, sinT, (T*)pool,
+                   (T*)q_nope, (T*)q_rot, gate, Ttok, H, dim, rot, rank, rot_dims, eps)));
+  return (int)hipGetLastError();
+}
+
+// LDS bytes the generic attention kernel needs for a chunk of KC keys
+int64_t dsv_latent_attn_lds(int dt, int rank, int rot, int KC) {
+  const int D = rank + rot;
+  return (int64_t)(HG * D + HG * KC + 3 * HG) * 4 + (int64_t)KC * (D | 1) * (dt == 0 ? 4 : 2);
+}
+
+int dsv_latent_attn(const void* q_lat, const void* q_rot, const void* pool, const int* tok_seq,
+                    const int* tok_pos, const int* table, int maxb, int bs, void* out,
+                    float* part, int dt, int Ttok, int H, int rank, int rot, int KC,
+                    int nsplit, float scale, hipStream_t s) {
+  if (rank > RPT * NT) return -1;
+  if (Ttok <= 0) return 0;
+  const int64_t lds = dsv_latent_attn_lds(dt, rank, rot, KC);
+  if (lds > 64 * 1024) return -2;
+  dim3 grid(Ttok, nsplit);
+  BY_DTYPE(dt, (latent_attn_k<T><<<grid, NT, lds, s>>>(
+                   (const T*)q_lat, (const T*)q_rot, (const T*)pool, tok_seq, tok_pos, table,
+                   maxb, bs, (T*)out, part, Ttok, H, rank, rot, KC, nsplit, scale)));
+  if (nsplit > 1) {
+    dim3 g2(Ttok, H);
+    BY_DTYPE(dt, (latent_attn_merge_k<T><<<g2, NT, 0, s>>>(part, (T*)out, Ttok, H, rank, nsplit)));
+  }
+  return (int)hipGetLastError();
+}
+
+int dsv_gate_merge(const void* o, const float* gate, void* out, int dt, int Ttok, int H, int v,
+                   hipStream_t s) {
+  const int64_t n = (int64_t)Ttok * H * v;
+  if (n <= 0) return 0;
+  BY_DTYPE(dt, (gate_merge_k<T><<<nblocks(n, 256), 256, 0, s>>>((const T*)o, gate, (T*)out, Ttok, H, v)));
+  return (int)hipGetLastError();
+}
+
+int dsv_xielu(const void* z, const float* pq, void* out, int dt, int64_t n, hipStream_t s) {
+  if (n <= 0) return 0;
+  BY_DTYPE(dt, (xielu_k<T><<<nblocks(n, 256), 256, 0, s>>>((const T*)z, pq, (T*)out, n)));
+  return (int)hipGetLastError();
+}
+
+int dsv_clamped_swiglu(const void* gu, void* out, int dt, int64_t rows, int F, float limit,
+                       hipStream_t s) {
+  if (rows * F <= 0) return 0;
+  BY_DTYPE(dt, (clamped_swiglu_k<T><<<nblocks(rows * F, 256), 256, 0, s>>>((const T*)gu, (T*)out, rows, F, limit)));
+  return (int)hipGetLastError();
+}
+
+int dsv_moe_combine(const void* y, const int64_t* inv, const float* w, const void* shared,
+                    const void* sg, void* out, int dt, int Ttok, int top, int C, hipStream_t s) {
+  if (Ttok <= 0) return 0;
+  BY_DTYPE(dt, (moe_combine_k<T><<<Ttok, 256, 0, s>>>((const T*)y, inv, w, (const T*)shared,
+                                                     (const T*)sg, (T*)out, top, C)));
+  return (int)hipGetLastError();
+}
+
+int dsv_topk_softmax(const float* z, int64_t* idx, float* w, int Ttok, int E, int top,
+                     hipStream_t s) {
+  if (Ttok <= 0) return 0;
+  topk_softmax_k<<<(Ttok + 63) / 64, 64, 0, s>>>(z, idx, w, Ttok, E, top);
+  return (int)hipGetLastError();
+}
+
+}  // extern "C"

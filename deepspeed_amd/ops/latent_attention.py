@@ -23,14 +23,19 @@ import torch
 from .rope import rope_interleaved_
 
 
+def _sk():
+    from . import serving_kernels
+    return serving_kernels
+
+
 def latent_prep(proj, batch, pool, norm_w, eps, heads, dim, rot, rank,
                 rot_dims, cos, sin):
     """proj [T, heads*(dim+rot) + rank + rot + heads] = q | latent | k_rot |
     gate logits. Writes the new rows into ``pool`` ([blocks, bs, rank+rot]).
     Returns q_nope [heads, T, dim] (contiguous), q_rot [T, heads, rot],
     gate [T, heads] fp32."""
-    if proj.is_cuda:
-        from . import serving_kernels as sk
+    if proj.is_cuda and _sk().enabled():
+        sk = _sk()
         return sk.latent_prep(proj, batch, pool, norm_w, eps, heads, dim, rot,
                               rank, rot_dims, cos, sin)
     T = proj.shape[0]
@@ -53,8 +58,8 @@ def latent_prep(proj, batch, pool, norm_w, eps, heads, dim, rot, rank,
 def latent_attention(q_lat, q_rot, pool, batch, rank, scale):
     """q_lat [heads, T, rank], q_rot [T, heads, rot]; pool holds every
     sequence's rows INCLUDING this step's. Returns [heads, T, rank]."""
-    if q_lat.is_cuda:
-        from . import serving_kernels as sk
+    if q_lat.is_cuda and _sk().enabled():
+        sk = _sk()
         return sk.latent_attention(q_lat, q_rot, pool, batch, rank, scale)
     bs = batch.block_size
     rows = pool.view(-1, pool.shape[-1])
@@ -82,8 +87,8 @@ def latent_attention(q_lat, q_rot, pool, batch, rank, scale):
 
 def gate_merge_heads(o, gate):
     """o [heads, T, v], gate [T, heads] fp32 -> [T, heads*v] (o's dtype)."""
-    if o.is_cuda:
-        from . import serving_kernels as sk
+    if o.is_cuda and _sk().enabled():
+        sk = _sk()
         return sk.gate_merge_heads(o, gate)
     H, T, v = o.shape
     return (o.float().transpose(0, 1) * gate[:, :, None]).to(o.dtype) \

@@ -137,17 +137,23 @@ class FusedLayerNorm(torch.nn.Module):
         return _LayerNormFn.apply(x, self.weight, self.bias, self.eps)
 
 
-def scalar_rms_norm(x, gain, eps=1e-6, out_dtype=None):
+def _sk():
+    from . import serving_kernels
+    return serving_kernels
+
+
+def scalar_rms_norm(x, gain, eps=1e-6, out_dtype=None, index=None):
     """RMS norm whose gain is ONE number for all coordinates:
     ``x * rsqrt(mean(x^2) + eps) * gain``. Statistics and the product are
     fp32 whatever ``x`` is; the result is rounded once to ``out_dtype``.
     x [T, C] (fp32 residual stream or 16-bit), gain a 0-d/1-element fp32
-    tensor."""
+    tensor. With ``index`` (int64 [R]) the rows ``x[index]`` are normed, the
+    gather fused into the kernel (embedding lookup, picking output rows)."""
     out_dtype = out_dtype or x.dtype
-    if x.is_cuda:
-        from . import serving_kernels as sk
-        return sk.scalar_rms_norm(x, gain, eps, out_dtype)
-    xf = x.float()
+    if x.is_cuda and _sk().enabled():
+        sk = _sk()
+        return sk.scalar_rms_norm(x.contiguous(), gain, eps, out_dtype, index)
+    xf = (x if index is None else x[index]).float()
     y = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) \
         * gain.float().reshape(())
     return y.to(out_dtype)
@@ -162,5 +168,5 @@ class ScalarRMSNorm(torch.nn.Module):
                                        requires_grad=False)
         self.eps = eps
 
-    def forward(self, x, out_dtype=None):
-        return scalar_rms_norm(x, self.gain, self.eps, out_dtype)
+    def forward(self, x, out_dtype=None, index=None):
+        return scalar_rms_norm(x, self.gain, self.eps, out_dtype, index)
