@@ -67,7 +67,7 @@ def latent_attention(q_lat, q_rot, pool, batch, rank, scale):
     at = 0
     for i, (st, cnt) in enumerate(zip(batch.starts, batch.counts)):
         L = st + cnt
-        pos = torch.arange(L)
+        pos = torch.arange(L, device=q_lat.device)
         ctx = rows[batch.block_table[i].long()[pos // bs] * bs + pos % bs]
         ctx = ctx.float()
         s = torch.einsum("htr,lr->htl", q_lat[:, at:at + cnt].float(),
@@ -75,7 +75,7 @@ def latent_attention(q_lat, q_rot, pool, batch, rank, scale):
         s = s + torch.einsum("thd,ld->htl", q_rot[at:at + cnt].float(),
                              ctx[:, rank:])
         s = s * scale
-        qpos = st + torch.arange(cnt)
+        qpos = st + torch.arange(cnt, device=q_lat.device)
         s = s.masked_fill(pos[None, None, :] > qpos[None, :, None],
                           float("-inf"))
         p = torch.softmax(s, -1)
