@@ -34,6 +34,13 @@ def parse_args():
                    help="ZeRO-Offload optimizer states to host DRAM")
     p.add_argument("--activation-checkpointing", action="store_true")
     p.add_argument("--local_rank", type=int, default=-1)
+    p.add_argument("--serving", type=str, default=None, choices=["fizesun"],
+                   help="instead of the training step: serving throughput "
+                        "(prefill, decode) of this design beside Llama at "
+                        "equal size, with per-kernel roofline distances")
+    p.add_argument("--serving-sizes", type=str, default="s,m,l")
+    p.add_argument("--serving-out", type=str, default=None,
+                   help="write the full serving report (JSON) here")
     return p.parse_args()
 
 
@@ -67,6 +74,10 @@ def build_model(name, world_size=1):
 
 def main():
     args = parse_args()
+    if args.serving:
+        from deepspeed_amd.inference.serving_bench import main as serving
+        serving(args.serving_sizes, args.serving_out)
+        return
     world_size = int(os.environ.get("WORLD_SIZE", 1))
     rank = int(os.environ.get("RANK", 0))
     os.environ.setdefault("MASTER_ADDR", "127.0.0.1")

@@ -1,0 +1,249 @@
+"""Serving throughput of Fizesun beside Llama at equal width, depth and
+feed-forward size, plus per-kernel distance from the roofline.
+
+Random weights, synthetic tokens, bf16, one GPU. For every size:
+* prefill: ``batch`` prompts of ``seq`` tokens in one ragged step (tokens/s);
+* decode: ``batch`` requests holding ``seq`` tokens, one token each per step;
+* kernels: each Fizesun kernel and the like kernel of the Llama path at the
+  same shapes, timed alone, against max(bytes / HBM bandwidth, flops / MFMA
+  peak). "distance" is measured time over that bound.
+Run through ``python bench.py --serving fizesun``.
+"""
+
+import json
+import time
+
+import torch
+
+HBM_BW = 8.0e12          # bytes/s
+MFMA_BF16 = 2.5e15       # flop/s dense
+
+SIZES = {
+    # width, layers, heads, ff, latent rank, rot, experts/top/expert ff
+    "s": dict(width=1024, layers=4, heads=8, ff=4096, rank=128, rot=32,
+              experts=8, top=2, eff=1024, batch=8, seq=1024),
+    "m": dict(width=2048, layers=4, heads=16, ff=8192, rank=256, rot=64,
+              experts=8, top=2, eff=2048, batch=8, seq=2048),
+    "l": dict(width=4096, layers=2, heads=32, ff=14336, rank=512, rot=64,
+              experts=8, top=2, eff=4096, batch=4, seq=4096),
+}
+
+
+def fizesun_config(z, vocab=32000):
+    mix = {"heads": z["heads"], "dim": 128, "rot_dim": z["rot"], "vdim": 128,
+           "kv_rank": z["rank"], "rot": {"base": 10000.0, "dims": z["rot"]},
+           "scale": (128 + z["rot"]) ** -0.5}
+    dense = {"kind": "dense", "ff": z["ff"]}
+    moe = {"kind": "moe", "expert": {"ff": z["eff"], "limit": 7.0},
+           "router": {"experts": z["experts"], "top": z["top"]},
+           "shared": {"ff": z["eff"], "limit": 7.0}}
+    layers = [{"type": "latent_attention", "mixer": mix,
+               "mlp": dense if i % 2 == 0 else moe}
+              for i in range(z["layers"])]
+    return {"architecture": "Fizesun", "vocab": vocab, "width": z["width"],
+            "norm": {"eps": 1e-6}, "canon": {"taps": 4}, "layers": layers}
+
+
+def _timed(fn, warmup=2, iters=5):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(iters):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / iters
+
+
+def _fizesun_throughput(z, dev):
+    from ..models.registry import build_model
+    from .ragged import ContinuousBatcher
+    model = build_model(fizesun_config(z), torch.bfloat16).init_random(0) \
+        .to(dev).eval()
+    B, S = z["batch"], z["seq"]
+    b = ContinuousBatcher(model, max_slots=B, dtype=torch.bfloat16,
+                          device=dev, max_tokens=B * (S + 64))
+    g = torch.Generator().manual_seed(0)
+    prompts = torch.randint(0, 32000, (B, S), generator=g).tolist()
+
+    def prefill():
+        reqs = [b.open(i) for i in range(B)]
+        b.feed([(r, p) for r, p in zip(reqs, prompts)], rows=[0])
+        return reqs
+
+    def prefill_and_close():
+        for r in prefill():
+            b.close(r)
+
+    t_pre = _timed(prefill_and_close, 1, 3)
+    reqs = prefill()
+
+    def decode():
+        b.feed([(r, [7]) for r in reqs], rows=list(range(B)))
+
+    t_dec = _timed(decode, 3, 20)
+    for r in reqs:
+        b.close(r)
+    del model, b
+    torch.cuda.empty_cache()
+    return {"prefill_tok_s": B * S / t_pre, "decode_tok_s": B / t_dec,
+            "decode_ms": 1e3 * t_dec}
+
+
+def _llama_throughput(z, dev):
+    from ..models import LlamaConfig, LlamaForCausalLM
+    from .ragged import ContinuousBatcher, PagedKVCache
+    B, S = z["batch"], z["seq"]
+    cfg = LlamaConfig(vocab_size=32000, hidden_size=z["width"],
+                      intermediate_size=z["ff"], num_layers=z["layers"],
+                      num_heads=z["heads"], num_kv_heads=max(1, z["heads"] // 4),
+                      max_seq_len=S + 64)
+    model = LlamaForCausalLM(cfg).to(torch.bfloat16).to(dev).eval()
+    b = ContinuousBatcher(model, max_slots=B, max_seq=S + 64,
+                          dtype=torch.bfloat16, device=dev,
+                          cache_cls=PagedKVCache)
+    g = torch.Generator().manual_seed(0)
+    ids = torch.randint(0, 32000, (B, S), generator=g).to(dev)
+    pos = torch.arange(S, dtype=torch.int32, device=dev).expand(B, S) \
+        .contiguous()
+    # prefill on the generate() path: contiguous cache, one batched forward
+    from .kv_cache import StaticKVCache
+    kv = StaticKVCache(cfg.num_layers, B, cfg.num_kv_heads, S + 64,
+                       cfg.head_dim, dtype=torch.bfloat16, device=dev)
+
+    @torch.no_grad()
+    def prefill():
+        kv.reset()
+        model(ids, positions=pos, kv_cache=kv)
+
+    t_pre = _timed(prefill, 1, 3)
+    del kv
+    last = torch.full((B, 1), 7, device=dev)
+
+    def decode():
+        for i in range(B):
+            b.cache.lens[i] = S
+        p = torch.full((B, 1), S, dtype=torch.int32, device=dev)
+        b._forward(last, list(range(B)), 1, p)
+
+    t_dec = _timed(decode, 3, 20)
+    del model, b
+    torch.cuda.empty_cache()
+    return {"prefill_tok_s": B * S / t_pre, "decode_tok_s": B / t_dec,
+            "decode_ms": 1e3 * t_dec}
+
+
+@torch.no_grad()
+def _kernel_rows(z, dev):
+    """(name, like, seconds, bound seconds) per kernel at this size."""
+    from ..ops import serving_kernels as sk
+    from ..ops.attention import flash_attn_available, flash_attn_fwd
+    from ..ops.norms import rms_norm
+    from ..ops.paged_attention import paged_decode_attention
+    from ..ops.swiglu import swiglu
+    from .state_cache import PagedStateCache
+    bf = torch.bfloat16
+    B, S, W, H = z["batch"], z["seq"], z["width"], z["heads"]
+    rank, rot, F = z["rank"], z["rot"], z["ff"]
+    T = B * S
+    out = []
+
+    def row(name, like, fn, nbytes, flops=0.0):
+        t = _timed(fn, 2, 5)
+        bound = max(nbytes / HBM_BW, flops / MFMA_BF16)
+        out.append({"kernel": name, "like": like, "us": 1e6 * t,
+                    "bound_us": 1e6 * bound, "distance": t / bound})
+
+    # ---- norm (+ conv) against RMSNorm
+    cache = PagedStateCache([rank + rot], {"conv": (1, 3, W)}, B,
+                            B * (S + 64), dtype=bf, device=dev)
+    x32 = torch.randn(T, W, device=dev)
+    x16 = x32.to(bf)
+    gain = torch.ones(1, device=dev)
+    cw = torch.randn(W, 4, device=dev).to(bf)
+    wn = torch.ones(W, device=dev, dtype=bf)
+    batch = cache.begin_ragged(list(range(B)), [S] * B)
+    row("norm_conv (fp32 stream in, bf16 out, 4 taps)", "rms_norm",
+        lambda: sk.norm_conv_ragged(x32, gain, 1e-6, cw,
+                                    cache.states["conv"][:, 0], batch, bf),
+        T * W * 6)
+    row("rms_norm (llama)", "", lambda: rms_norm(x16, wn, 1e-6), T * W * 4)
+    # ---- prefill attention
+    q_lat = (torch.randn(H, T, rank, device=dev) * 0.1).to(bf)
+    q_rot = (torch.randn(T, H, rot, device=dev) * 0.1).to(bf)
+    cache.pools[0].normal_()
+    fl = 2.0 * B * H * (S * S / 2) * (2 * rank + rot)
+    row("latent_attention prefill (MFMA tiles)", "flash_attn_fwd",
+        lambda: sk.latent_attention(q_lat, q_rot, cache.pools[0], batch, rank,
+                                    0.07, path="mfma"),
+        T * H * rank * 4 + T * (rank + rot) * 2, fl)
+    q = torch.randn(B, S, H, 128, device=dev).to(bf)
+    k = torch.randn(B, S, max(1, H // 4), 128, device=dev).to(bf)
+    if flash_attn_available(q, k):
+        row("flash_attn_fwd (llama)", "",
+            lambda: flash_attn_fwd(q, k, k, causal=True),
+            (2 * q.numel() + 2 * k.numel()) * 2,
+            4.0 * B * H * (S * S / 2) * 128)
+    cache.end_step()
+    # ---- decode attention
+    for i in range(B):
+        cache.lens[i] = S
+    batch = cache.begin_ragged(list(range(B)), [1] * B)
+    qd_lat, qd_rot = q_lat[:, :B].contiguous(), q_rot[:B].contiguous()
+    row("latent_attention decode (MFMA tiles, split keys)", "paged_decode",
+        lambda: sk.latent_attention(qd_lat, qd_rot, cache.pools[0], batch,
+                                    rank, 0.07),
+        B * (S + 1) * (rank + rot) * 2)
+    cache.end_step()
+    hkv = max(1, H // 4)
+    nb = B * ((S + 64) // 64)
+    kp = torch.randn(nb, hkv, 64, 128, device=dev).to(bf)
+    table = torch.arange(nb, dtype=torch.int32, device=dev).view(B, -1)
+    lens = torch.full((B,), S + 1, dtype=torch.int32, device=dev)
+    qd = torch.randn(B, H, 128, device=dev).to(bf)
+    row("paged_decode (llama)", "",
+        lambda: paged_decode_attention(qd, kp, kp, table, lens),
+        B * (S + 1) * hkv * 128 * 2 * 2)
+    # ---- activations
+    zf = torch.randn(T, F, device=dev).to(bf)
+    pq = torch.zeros(2, device=dev)
+    row("xielu", "swiglu", lambda: sk.xielu(zf, pq), T * F * 4)
+    gu = torch.randn(T, 2 * F, device=dev).to(bf)
+    row("clamped_swiglu", "swiglu", lambda: sk.clamped_swiglu(gu, 7.0),
+        T * F * 6)
+    up = torch.randn(T, F, device=dev).to(bf)
+    row("swiglu (llama)", "", lambda: swiglu(zf, up), T * F * 6)
+    return out
+
+
+def run(sizes=("s", "m", "l"), kernels=True):
+    dev = torch.device("cuda", torch.cuda.current_device())
+    report = {}
+    for name in sizes:
+        z = SIZES[name]
+        rec = {"size": {k: z[k] for k in z},
+               "fizesun": _fizesun_throughput(z, dev),
+               "llama": _llama_throughput(z, dev)}
+        if kernels:
+            rec["kernels"] = _kernel_rows(z, dev)
+        report[name] = rec
+        torch.cuda.empty_cache()
+    return report
+
+
+def main(sizes="s,m,l", out=None):
+    rep = run(tuple(sizes.split(",")))
+    if out:
+        with open(out, "w") as f:
+            json.dump(rep, f, indent=1)
+    best = rep[sizes.split(",")[-1]]
+    print(json.dumps({
+        "metric": "fizesun_serving_tokens_per_s", "unit": "tokens/s",
+        "dtype": "bf16", "data": "synthetic", "n_gpus": 1,
+        "value": best["fizesun"]["prefill_tok_s"], "higher_is_better": True,
+        "sizes": {k: {"fizesun": v["fizesun"], "llama": v["llama"],
+                      "worst_kernel_distance": max(
+                          (r["distance"] for r in v.get("kernels", [])
+                           if r["like"]), default=None)}
+                  for k, v in rep.items()}}))
+    return rep

@@ -87,6 +87,31 @@ class RoutedExperts(nn.Module):
         logits = F.linear(h.float(), self.router.float(),
                           self.router_bias.float())
         idx, weight = topk_softmax(logits, self.top)
+        picks = T * self.top
+        if picks <= self.DENSE_MAX_PICKS and 2 * picks >= self.experts:
+            # decode-sized steps: run every expert on every token as three
+            # batched GEMMs (the picks of a few tokens touch most experts'
+            # weights anyway) and pick the chosen outputs; no host round trip
+            mid = clamped_swiglu(torch.bmm(h.expand(self.experts, T, -1),
+                                           self.w_gu.transpose(1, 2)),
+                                 self.limit)
+            y = torch.bmm(mid, self.w_down.transpose(1, 2)) \
+                .reshape(self.experts * T, -1)
+            inv = idx * T + torch.arange(T, device=h.device)[:, None]
+        else:
+            y, inv = self._grouped(h, idx)
+        sh = sg = None
+        if self.shared is not None:
+            sh = self.shared(h)
+            sg = F.linear(h, self.shared_gate)
+        return moe_combine(y, inv, weight, sh, sg)
+
+    DENSE_MAX_PICKS = 64
+
+    def _grouped(self, h, idx):
+        """Tokens sorted by expert; one pair of GEMMs per expert that has
+        tokens. Returns the outputs in sorted order and each pick's place."""
+        T = h.shape[0]
         flat = idx.reshape(-1)
         order = torch.argsort(flat, stable=True)
         inv = torch.empty_like(order)
@@ -102,8 +127,4 @@ class RoutedExperts(nn.Module):
                                      self.limit)
                 y[at:at + n] = F.linear(mid, self.w_down[e])
                 at += n
-        sh = sg = None
-        if self.shared is not None:
-            sh = self.shared(h)
-            sg = F.linear(h, self.shared_gate)
-        return moe_combine(y, inv.view(T, self.top), weight, sh, sg)
+        return y, inv.view(T, self.top)

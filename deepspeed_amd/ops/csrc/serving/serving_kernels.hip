@@ -120,6 +120,77 @@ __global__ __launch_bounds__(NT) void norm_conv_k(
   }
 }
 
+// Tiled form for the usual short filters: a block owns CONV_TOKS consecutive
+// tokens, computes each row's norm factor once (one wave per row) and then
+// slides a register window over the tokens per channel, so a row of the
+// stream is read twice instead of once per tap.
+constexpr int CONV_TOKS = 8;
+
+template <typename T, int TAPS>
+__global__ __launch_bounds__(NT) void norm_conv_tile_k(
+    const float* __restrict__ x, const float* __restrict__ gain,
+    const T* __restrict__ w, const T* __restrict__ state,
+    int64_t state_slot_stride, const int* __restrict__ cu,
+    const int* __restrict__ seq_slot, const int* __restrict__ tok_seq,
+    const int* __restrict__ tok_pos, T* __restrict__ out, int Ttok, int C,
+    float eps) {
+  constexpr int TAIL = TAPS - 1;
+  constexpr int NR = CONV_TOKS + TAIL;
+  __shared__ float rinv[NR];
+  const int t0 = blockIdx.x * CONV_TOKS;
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+  const float g = gain[0];
+  for (int ri = wid; ri < NR; ri += NT / 64) {
+    const int tt = t0 - TAIL + ri;
+    float ss = 0.f;
+    if (tt >= 0 && tt < Ttok) {
+      const float* row = x + (int64_t)tt * C;
+      for (int c = lane; c < C; c += 64) ss += row[c] * row[c];
+    }
+    ss = wave_sum(ss);
+    if (lane == 0) rinv[ri] = rsqrtf(ss / (float)C + eps) * g;
+  }
+  __syncthreads();
+  for (int c = threadIdx.x; c < C; c += NT) {
+    float wv[TAPS];
+#pragma unroll
+    for (int k = 0; k < TAPS; ++k) wv[k] = ld(w + (int64_t)c * TAPS + k);
+    float win[TAIL > 0 ? TAIL : 1];  // win[k-1]: input k tokens back (flat order)
+#pragma unroll
+    for (int k = 1; k <= TAIL; ++k) {
+      const int tt = t0 - k;
+      win[k - 1] = tt >= 0 ? rnd<T>(x[(int64_t)tt * C + c] * rinv[TAIL - k]) : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < CONV_TOKS; ++i) {
+      const int t = t0 + i;
+      if (t < Ttok) {
+        const int s = tok_seq[t];
+        const int j = t - cu[s];
+        const int pos = tok_pos[t];
+        const T* sl = state + (int64_t)seq_slot[s] * state_slot_stride;
+        const float h0 = rnd<T>(x[(int64_t)t * C + c] * rinv[TAIL + i]);
+        float acc = wv[TAIL] * h0;
+#pragma unroll
+        for (int k = 1; k <= TAIL; ++k) {
+          float hk;
+          if (k <= j)
+            hk = win[k - 1];
+          else if (pos - k < 0)
+            hk = 0.f;
+          else
+            hk = ld(sl + (int64_t)(TAIL + j - k) * C + c);
+          acc += wv[TAIL - k] * hk;
+        }
+        st(out + (int64_t)t * C + c, h0 + acc);
+#pragma unroll
+        for (int k = TAIL; k >= 2; --k) win[k - 1] = win[k - 2];
+        if (TAIL > 0) win[0] = h0;
+      }
+    }
+  }
+}
+
 // One block per sequence: the tail becomes the last taps-1 normed inputs.
 template <typename T>
 __global__ __launch_bounds__(NT) void conv_tail_k(
@@ -397,6 +468,277 @@ __global__ __launch_bounds__(NT) void latent_attn_merge_k(
   }
 }
 
+// ------------------------------------------- latent attention, MFMA tiles
+// bf16 prefill path. The rows of one sequence's step are (token, head) pairs,
+// token-major: row m belongs to token m / H and sees keys 0..start + m / H, so
+// all heads of a token share its key range and the whole step is one
+// [count*H, Dk] x [Dk, keys] product per sequence. A workgroup of 4 waves owns
+// 128 rows (32 per wave) and walks the keys 32 at a time:
+//   S^T[key, row] = mfma(A = K tile from LDS, B = Q fragments in registers)
+//   online softmax per row (one row per lane pair, fp32)
+//   O^T[d, row]  += mfma(A = V^T tile from LDS, B = P fragments)
+// mfma_f32_32x32x16_bf16 layouts: A row = lane&31, k = reg + 8*(lane>>5);
+// B col = lane&31, k = reg + 8*(lane>>5); C/D col = lane&31,
+// row = (reg&3) + 8*(reg>>2) + 4*(lane>>5).
+typedef short bf16x8s __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ short f2bf_bits(float f) {
+  union { float f; unsigned u; } c;
+  c.f = f;
+  return (short)((c.u + 0x7FFF + ((c.u >> 16) & 1)) >> 16);
+}
+
+constexpr int TB_ROWS = 128;  // rows per workgroup
+constexpr int TB_KEYS = 32;   // keys per step
+constexpr int VT_STRIDE = TB_KEYS + 8;
+
+// SPLIT = 2: two waves share a row block and each keeps half of the output
+// columns (the score product is computed twice) so that wide latents fit the
+// register file; the workgroup then owns 64 rows.
+template <int DVB, int DKT_MAX, int SPLIT, bool PREFETCH>
+__global__ __launch_bounds__(256) void latent_attn_mfma_k(
+    const short* __restrict__ q_lat,  // [H, Ttok, rank]
+    const short* __restrict__ q_rot,  // [Ttok, H, rot]
+    const short* __restrict__ pool, const int* __restrict__ work,
+    const int* __restrict__ cu, const int* __restrict__ seq_start,
+    const int* __restrict__ table, int maxb, int bs, bf16* __restrict__ out,
+    float* __restrict__ part,  // [Ttok, nsplit, H, rank + 2] when nsplit > 1
+    int Ttok, int H, int rank, int rot, int nsplit, float scale) {
+  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+  constexpr int DVW = DVB / SPLIT;     // output blocks of this wave
+  constexpr int ROWS = TB_ROWS / SPLIT;
+  constexpr int CPT = (DKT_MAX + 3) / 4;  // staged 16-byte chunks per thread
+  const int Dk = rank + rot;
+  const int DkP = (Dk + 15) & ~15;
+  const int DKT = DkP >> 4;
+  const int KSS = DkP + 8;
+  short* Ks = reinterpret_cast<short*>(smem_raw);  // [TB_KEYS][KSS]
+  short* Vt = Ks + TB_KEYS * KSS;                  // [DVB*32][VT_STRIDE]
+  const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
+  const int hl = lane >> 5, l31 = lane & 31;
+  const int s = work[2 * blockIdx.x], m0 = work[2 * blockIdx.x + 1];
+  const int split = blockIdx.y;
+  const int count = cu[s + 1] - cu[s], start = seq_start[s];
+  const int rows = count * H;
+  const int part_id = wid % SPLIT;
+  const int m_raw = m0 + (wid / SPLIT) * 32 + l31;
+  const int m = min(m_raw, rows - 1);
+  const int j = m / H, h = m - j * H;
+  const int t = cu[s] + j;
+  const int qpos = start + j;
+  const int kmax = start + min(m0 + ROWS - 1, rows - 1) / H;  // inclusive
+  const int* tab = table + (int64_t)s * maxb;
+  // this split's key steps
+  const int nsteps = kmax / TB_KEYS + 1;
+  const int per = (nsteps + nsplit - 1) / nsplit;
+  const int s_lo = split * per, s_hi = min(nsteps, s_lo + per);
+  float* pp = nullptr;
+  if (nsplit > 1)
+    pp = part + (((int64_t)t * nsplit + split) * H + h) * (rank + 2);
+  if (s_lo >= s_hi) {  // block-uniform: nothing to see in this split
+    if (m_raw < rows && part_id == 0 && hl == 0) {
+      pp[0] = -INFINITY;
+      pp[1] = 0.f;
+    }
+    return;
+  }
+
+  bf16x8s qf[DKT_MAX];
+#pragma unroll
+  for (int kt = 0; kt < DKT_MAX; ++kt) {
+    if (kt < DKT) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int d = 16 * kt + 8 * hl + e;
+        short v = 0;
+        if (d < rank)
+          v = q_lat[((int64_t)h * Ttok + t) * rank + d];
+        else if (d < Dk)
+          v = q_rot[((int64_t)t * H + h) * rot + d - rank];
+        qf[kt][e] = v;
+      }
+    }
+  }
+  f32x16 oacc[DVW];
+#pragma unroll
+  for (int db = 0; db < DVW; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
+  float mrun = -INFINITY, lrun = 0.f;
+  const int cpk = DkP >> 3;  // 8-element chunks per key
+  const bool vec_ok = (Dk & 7) == 0;
+
+  // Staging: chunk c of a tile is (dims 8*(c>>5).., key c&31): neighbouring
+  // lanes take neighbouring keys, so the transposed writes fall into one row.
+  auto fetch_one = [&](int i, int k0) -> bf16x8s {
+    const int c = tid + i * 256;
+    bf16x8s v;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = 0;
+    if (c < TB_KEYS * cpk) {
+      const int ch = c >> 5, key = c & 31;
+      const int p = k0 + key;
+      if (p <= kmax) {
+        const int64_t row = (int64_t)tab[p / bs] * bs + p % bs;
+        const short* src = pool + row * Dk + ch * 8;
+        if (vec_ok && ch * 8 + 8 <= Dk) {
+          v = *reinterpret_cast<const bf16x8s*>(src);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (ch * 8 + e < Dk) v[e] = src[e];
+        }
+      }
+    }
+    return v;
+  };
+  auto stash_one = [&](int i, const bf16x8s& v) {
+    const int c = tid + i * 256;
+    if (c < TB_KEYS * cpk) {
+      const int ch = c >> 5, key = c & 31;
+      *reinterpret_cast<bf16x8s*>(Ks + key * KSS + ch * 8) = v;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int d = ch * 8 + e;
+        if (d < DVB * 32) Vt[d * VT_STRIDE + key] = d < rank ? v[e] : (short)0;
+      }
+    }
+  };
+  bf16x8s pre[PREFETCH ? CPT : 1];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < CPT; ++i)
+      if (PREFETCH) pre[i] = fetch_one(i, k0);
+  };
+  auto stash = [&](int k0) {
+    if (PREFETCH) {
+#pragma unroll
+      for (int i = 0; i < CPT; ++i) stash_one(i, pre[i]);
+    } else {
+#pragma unroll 1
+      for (int i = 0; i < CPT; ++i) stash_one(i, fetch_one(i, k0));
+    }
+  };
+
+  // PREFETCH keeps the next tile's loads in flight during the products; the
+  // widest class has no registers to spare for that
+  if (PREFETCH) fetch(s_lo * TB_KEYS);
+  for (int step = s_lo; step < s_hi; ++step) {
+    const int k0 = step * TB_KEYS;
+    __syncthreads();
+    stash(k0);
+    __syncthreads();
+    if (PREFETCH && step + 1 < s_hi) fetch(k0 + TB_KEYS);
+    f32x16 st;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) st[r] = 0.f;
+#pragma unroll
+    for (int kt = 0; kt < DKT_MAX; ++kt) {
+      if (kt < DKT) {
+        const bf16x8s kf =
+            *reinterpret_cast<const bf16x8s*>(Ks + l31 * KSS + 16 * kt + 8 * hl);
+        st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kt], st, 0, 0, 0);
+      }
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int key = k0 + (r & 3) + 8 * (r >> 2) + 4 * hl;
+      const float v = key <= qpos ? st[r] * scale : -INFINITY;
+      st[r] = v;
+      mx = fmaxf(mx, v);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(mrun, mx);
+    // a row that has seen no key yet (a later split of an early token) keeps
+    // weight zero without producing inf - inf
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = expf(mrun - m_use);
+    float psum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float p = expf(st[r] - m_use);
+      st[r] = p;
+      psum += p;
+    }
+    psum += __shfl_xor(psum, 32, 64);
+    lrun = lrun * alpha + psum;
+    mrun = m_new;
+#pragma unroll
+    for (int db = 0; db < DVW; ++db)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      // B fragment of P: keys 16*ks + 8*hl + 0..7 of this lane's row; half of
+      // them sit in the partner lane (lane ^ 32)
+      bf16x8s pf;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float a0 = st[i + 8 * ks], a1 = st[i + 8 * ks + 4];
+        const float recv = __shfl_xor(hl ? a0 : a1, 32, 64);
+        pf[i] = f2bf_bits(hl ? recv : a0);
+        pf[i + 4] = f2bf_bits(hl ? a1 : recv);
+      }
+#pragma unroll
+      for (int db = 0; db < DVW; ++db) {
+        const bf16x8s vf = *reinterpret_cast<const bf16x8s*>(
+            Vt + (32 * (part_id * DVW + db) + l31) * VT_STRIDE + 16 * ks + 8 * hl);
+        oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf, oacc[db], 0, 0, 0);
+      }
+    }
+  }
+  if (m_raw < rows) {
+    if (nsplit > 1) {
+      if (part_id == 0 && hl == 0) {
+        pp[0] = mrun;
+        pp[1] = lrun;
+      }
+#pragma unroll
+      for (int db = 0; db < DVW; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int d = 32 * (part_id * DVW + db) + (r & 3) + 8 * (r >> 2) + 4 * hl;
+          if (d < rank) pp[2 + d] = oacc[db][r];
+        }
+    } else {
+      const float inv = 1.f / lrun;
+      bf16* o = out + ((int64_t)h * Ttok + t) * rank;
+#pragma unroll
+      for (int db = 0; db < DVW; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int d = 32 * (part_id * DVW + db) + (r & 3) + 8 * (r >> 2) + 4 * hl;
+          if (d < rank) o[d] = __float2bfloat16(oacc[db][r] * inv);
+        }
+    }
+  }
+}
+
+template <int DVB, int DKT_MAX, int SPLIT, bool PREFETCH>
+int launch_latent_attn_mfma(const void* q_lat, const void* q_rot, const void* pool,
+                            const int* work, int nwork, const int* cu, const int* seq_start,
+                            const int* table, int maxb, int bs, void* out, float* part,
+                            int Ttok, int H, int rank, int rot, int nsplit, float scale,
+                            hipStream_t s) {
+  const int DkP = (rank + rot + 15) & ~15;
+  const size_t lds = (size_t)TB_KEYS * (DkP + 8) * 2 + (size_t)DVB * 32 * VT_STRIDE * 2;
+  auto kern = latent_attn_mfma_k<DVB, DKT_MAX, SPLIT, PREFETCH>;
+  if (lds > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+  }
+  kern<<<dim3(nwork, nsplit), 256, lds, s>>>((const short*)q_lat, (const short*)q_rot,
+                                             (const short*)pool, work, cu, seq_start, table, maxb,
+                                             bs, (bf16*)out, part, Ttok, H, rank, rot, nsplit,
+                                             scale);
+  if (nsplit > 1)
+    latent_attn_merge_k<bf16><<<dim3(Ttok, H), NT, 0, s>>>(part, (bf16*)out, Ttok, H, rank, nsplit);
+  return (int)hipGetLastError();
+}
+
 // out[t, h*v + c] = o[h, t, c] * gate[t, h]
 template <typename T>
 __global__ void gate_merge_k(const T* __restrict__ o, const float* __restrict__ gate,
@@ -528,9 +870,29 @@ int dsv_norm_conv(const float* x, const float* gain, const void* w, void* state,
                   int dt, int Ttok, int nseq, int C, int taps, float eps, hipStream_t s) {
   if (taps > MAXTAPS) return -1;
   if (Ttok <= 0) return 0;
-  BY_DTYPE(dt, (norm_conv_k<T><<<Ttok, NT, 0, s>>>(x, gain, (const T*)w, (const T*)state,
-                                                    state_slot_stride, cu, seq_slot, tok_seq,
-                                                    tok_pos, (T*)out, C, taps, eps)));
+  const int tiles = (Ttok + CONV_TOKS - 1) / CONV_TOKS;
+#define TILE(N)                                                                              \
+  case N:                                                                                    \
+    BY_DTYPE(dt, (norm_conv_tile_k<T, N><<<tiles, NT, 0, s>>>(                               \
+                     x, gain, (const T*)w, (const T*)state, state_slot_stride, cu, seq_slot, \
+                     tok_seq, tok_pos, (T*)out, Ttok, C, eps)));                             \
+    break
+  switch (taps) {
+    TILE(1);
+    TILE(2);
+    TILE(3);
+    TILE(4);
+    TILE(5);
+    TILE(6);
+    TILE(7);
+    TILE(8);
+    default:
+      BY_DTYPE(dt, (norm_conv_k<T><<<Ttok, NT, 0, s>>>(x, gain, (const T*)w, (const T*)state,
+                                                        state_slot_stride, cu, seq_slot,
+                                                        tok_seq, tok_pos, (T*)out, C, taps,
+                                                        eps)));
+  }
+#undef TILE
   if (taps > 1)
     BY_DTYPE(dt, (conv_tail_k<T><<<nseq, NT, 0, s>>>(x, gain, (T*)state, state_slot_stride, cu,
                                                       seq_slot, seq_start, C, taps, eps)));
@@ -571,6 +933,36 @@ int dsv_latent_attn(const void* q_lat, const void* q_rot, const void* pool, cons
     BY_DTYPE(dt, (latent_attn_merge_k<T><<<g2, NT, 0, s>>>(part, (T*)out, Ttok, H, rank, nsplit)));
   }
   return (int)hipGetLastError();
+}
+
+// 1 when the MFMA tile kernel covers these sizes (bf16 only)
+int dsv_latent_attn_mfma_ok(int rank, int rot) {
+  return rank >= 1 && rank <= 512 && rank + rot <= 640;
+}
+
+// rows of a sequence's count*H that one workgroup takes
+int dsv_latent_attn_mfma_rows(int rank, int rot) {
+  return (rank <= 256 && rank + rot <= 320) ? TB_ROWS : TB_ROWS / 2;
+}
+
+// work: [nwork][2] = (sequence, first row of a tile of its count*H rows)
+int dsv_latent_attn_mfma(const void* q_lat, const void* q_rot, const void* pool, const int* work,
+                         int nwork, const int* cu, const int* seq_start, const int* table,
+                         int maxb, int bs, void* out, float* part, int Ttok, int H, int rank,
+                         int rot, int nsplit, float scale, hipStream_t s) {
+  if (!dsv_latent_attn_mfma_ok(rank, rot)) return -1;
+  if (nsplit < 1 || (nsplit > 1 && !part)) return -3;
+  if (nwork <= 0) return 0;
+  const int dk = rank + rot;
+#define GO(DVB, DKT, SPLIT, PF) \
+  return launch_latent_attn_mfma<DVB, DKT, SPLIT, PF>(q_lat, q_rot, pool, work, nwork, cu, seq_start, \
+                                           table, maxb, bs, out, part, Ttok, H, rank, rot, \
+                                           nsplit, scale, s)
+  if (rank <= 64 && dk <= 128) GO(2, 8, 1, true);
+  if (rank <= 128 && dk <= 192) GO(4, 12, 1, true);
+  if (rank <= 256 && dk <= 320) GO(8, 20, 1, true);
+  GO(16, 40, 2, false);
+#undef GO
 }
 
 int dsv_gate_merge(const void* o, const float* gate, void* out, int dt, int Ttok, int H, int v,

@@ -175,20 +175,63 @@ def _attn_plan(batch, dtype, rank, rot):
     return kc, nsplit
 
 
-def latent_attention(q_lat, q_rot, pool, batch, rank, scale):
+def _tile_work(batch, heads, tile_rows, device):
+    """[(sequence, first row)] over every sequence's count*heads rows, late
+    (long-history) tiles first so the heavy workgroups start early."""
+    key = ("latent_tiles", heads, tile_rows)
+    if key not in batch.extra:
+        import numpy as np
+        work = []
+        for i, (st, c) in enumerate(zip(batch.starts, batch.counts)):
+            for m0 in range(0, c * heads, tile_rows):
+                work.append((st + (m0 + tile_rows) // heads, i, m0))
+        work.sort(reverse=True)
+        arr = np.asarray([(i, m0) for _, i, m0 in work], np.int32).reshape(-1)
+        batch.extra[key] = (torch.from_numpy(arr).to(device), len(work))
+    return batch.extra[key]
+
+
+def latent_attention(q_lat, q_rot, pool, batch, rank, scale, path=None):
+    """``path`` forces "mfma" or "exact" (tests); default chooses by size."""
     H, T, r = q_lat.shape
     rot = q_rot.shape[2]
     assert r == rank and q_rot.shape[:2] == (T, H) and T == batch.n_tokens
     assert pool.shape[-1] == rank + rot and pool.shape[1] == batch.block_size
     assert q_lat.dtype == pool.dtype == q_rot.dtype
+    assert q_rot.is_contiguous() and pool.is_contiguous()
     q_lat = q_lat.contiguous()
-    kc, nsplit = _attn_plan(batch, q_lat.dtype, rank, rot)
+    lib = load()
     out = torch.empty_like(q_lat)
+    mfma = q_lat.dtype == torch.bfloat16 and \
+        lib.dsv_latent_attn_mfma_ok(_i(rank), _i(rot)) == 1
+    if path is None:
+        path = "mfma" if mfma else "exact"
+    if path == "mfma":
+        assert mfma, "the MFMA kernel is bf16 and bounded in rank"
+        rows = lib.dsv_latent_attn_mfma_rows(_i(rank), _i(rot))
+        work, n = _tile_work(batch, H, rows, q_lat.device)
+        # few tiles over long histories (decoding): split the keys so the
+        # launch still covers the chip; partial sums are merged in fp32
+        nsplit = 1
+        if n < 128:
+            nsplit = max(1, min(32, batch.max_ctx // 128, 512 // n))
+        part = None
+        if nsplit > 1:
+            part = torch.empty(T, nsplit, H, rank + 2, dtype=torch.float32,
+                               device=q_lat.device)
+        _check(lib.dsv_latent_attn_mfma(
+            _p(q_lat), _p(q_rot), _p(pool), _p(work), _i(n), _p(batch.cu),
+            _p(batch.seq_start), _p(batch.block_table),
+            _i(batch.block_table.shape[1]), _i(batch.block_size), _p(out),
+            _p(part), _i(T), _i(H), _i(rank), _i(rot), _i(nsplit), _f(scale),
+            _stream()), "latent_attention(mfma)")
+        return out
+    kc, nsplit = _attn_plan(batch, q_lat.dtype, rank, rot)
     part = None
     if nsplit > 1:
         part = torch.empty(T, nsplit, H, rank + 2, dtype=torch.float32,
                            device=q_lat.device)
-    _check(load().dsv_latent_attn(
+    _check(lib.dsv_latent_attn(
         _p(q_lat), _p(q_rot), _p(pool), _p(batch.tok_seq), _p(batch.tok_pos),
         _p(batch.block_table), _i(batch.block_table.shape[1]),
         _i(batch.block_size), _p(out), _p(part), _i(_dt(q_lat)), _i(T), _i(H),

@@ -167,13 +167,19 @@ def close_rms(got, want, tol):
 def test_norm_conv_matches_oracle_over_cuts():
     from deepspeed_amd.ops.causal_conv import norm_conv_ragged
     torch.manual_seed(0)
-    C, taps, S = 10, 4, 9
+    _norm_conv_case(4)
+    _norm_conv_case(9)      # longer than the filters the tiled kernel covers
+
+
+def _norm_conv_case(taps):
+    from deepspeed_amd.ops.causal_conv import norm_conv_ragged
+    C, S = 10, 9
     x = torch.randn(S, C) * 3
     g, w = torch.tensor([1.3]), torch.randn(C, taps) * 0.5
     want = O.with_input_conv(O.scalar_norm(x.double(), g.double(), 1e-5),
                              w.double())
     for cuts in ([9], [1] * 9, [2, 5, 1, 1], [4, 2, 3]):
-        cache = PagedStateCache([4], {"conv": (1, taps - 1, C)}, 2, 64,
+        cache = PagedStateCache([4], {"conv": (3, taps - 1, C)}, 2, 64,
                                 block_size=8, device=DEV)
         cache.reset_slot(1)
         got, at = [], 0
@@ -181,7 +187,7 @@ def test_norm_conv_matches_oracle_over_cuts():
             b = cache.begin_ragged([1], [c])
             got.append(norm_conv_ragged(x[at:at + c].to(DEV).contiguous(),
                                         g.to(DEV), 1e-5, w.to(DEV),
-                                        cache.states["conv"][:, 0], b,
+                                        cache.states["conv"][:, 1], b,
                                         torch.float32).cpu())
             cache.end_step()
             at += c
@@ -228,10 +234,13 @@ def test_clamped_expert_limits_bite():
 
 @pytest.mark.parametrize("experts,top,shared", [(5, 2, True), (4, 4, False),
                                                  (3, 1, True)])
-def test_routed_experts_match_oracle(experts, top, shared):
+@pytest.mark.parametrize("grouped", [False, True])
+def test_routed_experts_match_oracle(experts, top, shared, grouped):
     cfg = config([(mixer(), moe(experts, top, shared=shared))])
     s = Served(cfg)
     layer = s.model.layers[0].mlp
+    if grouped:                      # the path of large steps: tokens by expert
+        layer.DENSE_MAX_PICKS = 0
     torch.manual_seed(3)
     h = torch.randn(11, cfg["width"])
     want = O.moe_ff(h.double(), s.w64, "l0.mlp.", cfg["layers"][0]["mlp"])
@@ -562,3 +571,35 @@ def test_split_key_decode_over_long_history():
     t = toks(1500, seed=13)
     got = s.run(t, [1490] + [1] * 10)[-10:]
     close(got, s.oracle(t)[-10:], 5e-4)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("heads,rank,rot", [(3, 20, 6), (7, 56, 8),
+                                            (5, 96, 32), (4, 200, 40),
+                                            (2, 512, 64)])
+def test_mfma_tiles_match_the_exact_kernel(heads, rank, rot):
+    """Ragged batch (held tokens, portions of unequal length, a single decoded
+    token) over 16-token blocks handed out in scrambled order."""
+    from deepspeed_amd.ops import serving_kernels as sk
+    g = torch.Generator().manual_seed(rank)
+    bs = 16
+    cache = PagedStateCache([rank + rot], {}, 4, 2048, block_size=bs,
+                            dtype=torch.bfloat16, device=DEV)
+    perm = torch.randperm(cache.num_blocks, generator=g).tolist()
+    cache.free_blocks = perm
+    held, counts = [0, 37, 300, 129], [150, 1, 77, 200]
+    for slot, n in enumerate(held):
+        cache.lens[slot] = n
+    b = cache.begin_ragged([0, 1, 2, 3], counts)
+    cache.pools[0].copy_(torch.randn(cache.pools[0].shape, generator=g))
+    T = sum(counts)
+    q_lat = (torch.randn(heads, T, rank, generator=g) * 0.3).to(
+        DEV, torch.bfloat16)
+    q_rot = torch.randn(T, heads, rot, generator=g).to(DEV, torch.bfloat16)
+    a = sk.latent_attention(q_lat, q_rot, cache.pools[0], b, rank, 0.2,
+                            path="mfma").float().cpu()
+    e = sk.latent_attention(q_lat, q_rot, cache.pools[0], b, rank, 0.2,
+                            path="exact").float().cpu()
+    # the weights are rounded to 16 bits before the second product
+    assert (a - e).abs().max().item() < 0.03
+    assert ((a - e) ** 2).mean().sqrt().item() < 0.004
