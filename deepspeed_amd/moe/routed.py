@@ -30,8 +30,8 @@ def topk_softmax(logits, top):
 
 
 def moe_combine(y, inv, weight, shared=None, shared_gate=None):
-    """y [T*top, C] expert outputs in expert-sorted order; inv [T, top] the
-    sorted position of each (token, choice); weight [T, top] fp32. Returns
+    """y [N, C] expert outputs; inv [T, top] the row of y that holds each
+    (token, choice); weight [T, top] fp32. Returns
     sum_k weight[t, k] * y[inv[t, k]] (+ sigmoid(shared_gate[t]) *
     shared[t]) as [T, C] in y's dtype."""
     if y.is_cuda and _sk().enabled():

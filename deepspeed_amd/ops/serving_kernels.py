@@ -273,7 +273,7 @@ def clamped_swiglu(gu, limit):
 def moe_combine(y, inv, weight, shared=None, shared_gate=None):
     T, top = inv.shape
     C = y.shape[1]
-    assert y.shape[0] == T * top and weight.shape == (T, top)
+    assert y.shape[0] >= T * top and weight.shape == (T, top)
     assert inv.dtype == torch.int64 and weight.dtype == torch.float32
     if shared is not None:
         assert shared.shape == (T, C) and shared_gate.numel() == T
