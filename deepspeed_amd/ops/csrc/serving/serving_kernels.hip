@@ -28,6 +28,12 @@ template <> __device__ __forceinline__ float rnd<bf16>(float v) {
   return __bfloat162float(__float2bfloat16(v));
 }
 
+__device__ __forceinline__ short f2bf_bits(float f) {
+  union { float f; unsigned u; } c;
+  c.f = f;
+  return (short)((c.u + 0x7FFF + ((c.u >> 16) & 1)) >> 16);
+}
+
 __device__ __forceinline__ float wave_sum(float x) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o, 64);
@@ -126,7 +132,39 @@ __global__ __launch_bounds__(NT) void norm_conv_k(
 // stream is read twice instead of once per tap.
 constexpr int CONV_TOKS = 8;
 
-template <typename T, int TAPS>
+template <int VEC>
+__device__ __forceinline__ void ld_vec(const float* p, float (&v)[VEC]) {
+  if (VEC == 4) {
+    const float4 q = *reinterpret_cast<const float4*>(p);
+    v[0] = q.x; v[1] = q.y; v[2] = q.z; v[VEC - 1] = q.w;
+  } else {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) v[i] = p[i];
+  }
+}
+template <int VEC>
+__device__ __forceinline__ void st_vec(float* p, const float (&v)[VEC]) {
+  if (VEC == 4) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[VEC - 1]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) p[i] = v[i];
+  }
+}
+template <int VEC>
+__device__ __forceinline__ void st_vec(bf16* p, const float (&v)[VEC]) {
+  if (VEC == 4) {
+    uint2 q;
+    q.x = (unsigned short)f2bf_bits(v[0]) | ((unsigned)(unsigned short)f2bf_bits(v[1]) << 16);
+    q.y = (unsigned short)f2bf_bits(v[2]) | ((unsigned)(unsigned short)f2bf_bits(v[VEC - 1]) << 16);
+    *reinterpret_cast<uint2*>(p) = q;
+  } else {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) p[i] = __float2bfloat16(v[i]);
+  }
+}
+
+template <typename T, int TAPS, int VEC>
 __global__ __launch_bounds__(NT) void norm_conv_tile_k(
     const float* __restrict__ x, const float* __restrict__ gain,
     const T* __restrict__ w, const T* __restrict__ state,
@@ -137,55 +175,93 @@ __global__ __launch_bounds__(NT) void norm_conv_tile_k(
   constexpr int TAIL = TAPS - 1;
   constexpr int NR = CONV_TOKS + TAIL;
   __shared__ float rinv[NR];
+  __shared__ int meta[CONV_TOKS][3];  // offset in its sequence's step, position, slot
   const int t0 = blockIdx.x * CONV_TOKS;
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
   const float g = gain[0];
+  if (threadIdx.x < CONV_TOKS && t0 + threadIdx.x < Ttok) {
+    const int t = t0 + threadIdx.x, s = tok_seq[t];
+    meta[threadIdx.x][0] = t - cu[s];
+    meta[threadIdx.x][1] = tok_pos[t];
+    meta[threadIdx.x][2] = seq_slot[s];
+  }
   for (int ri = wid; ri < NR; ri += NT / 64) {
     const int tt = t0 - TAIL + ri;
     float ss = 0.f;
     if (tt >= 0 && tt < Ttok) {
       const float* row = x + (int64_t)tt * C;
-      for (int c = lane; c < C; c += 64) ss += row[c] * row[c];
+      for (int c = lane * VEC; c < C; c += 64 * VEC) {
+        float v[VEC];
+        ld_vec<VEC>(row + c, v);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) ss += v[i] * v[i];
+      }
     }
     ss = wave_sum(ss);
     if (lane == 0) rinv[ri] = rsqrtf(ss / (float)C + eps) * g;
   }
   __syncthreads();
-  for (int c = threadIdx.x; c < C; c += NT) {
-    float wv[TAPS];
+  for (int c = threadIdx.x * VEC; c < C; c += NT * VEC) {
+    float wv[VEC][TAPS];
 #pragma unroll
-    for (int k = 0; k < TAPS; ++k) wv[k] = ld(w + (int64_t)c * TAPS + k);
-    float win[TAIL > 0 ? TAIL : 1];  // win[k-1]: input k tokens back (flat order)
+    for (int v = 0; v < VEC; ++v)
+#pragma unroll
+      for (int k = 0; k < TAPS; ++k) wv[v][k] = ld(w + (int64_t)(c + v) * TAPS + k);
+    float win[TAIL > 0 ? TAIL : 1][VEC];  // win[k-1]: input k tokens back (flat order)
 #pragma unroll
     for (int k = 1; k <= TAIL; ++k) {
       const int tt = t0 - k;
-      win[k - 1] = tt >= 0 ? rnd<T>(x[(int64_t)tt * C + c] * rinv[TAIL - k]) : 0.f;
+      float xv[VEC];
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) xv[v] = 0.f;
+      if (tt >= 0) ld_vec<VEC>(x + (int64_t)tt * C + c, xv);
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) win[k - 1][v] = rnd<T>(xv[v] * rinv[TAIL - k]);
+    }
+    float xs[CONV_TOKS][VEC];
+#pragma unroll
+    for (int i = 0; i < CONV_TOKS; ++i) {
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) xs[i][v] = 0.f;
+      if (t0 + i < Ttok) ld_vec<VEC>(x + (int64_t)(t0 + i) * C + c, xs[i]);
     }
 #pragma unroll
     for (int i = 0; i < CONV_TOKS; ++i) {
       const int t = t0 + i;
       if (t < Ttok) {
-        const int s = tok_seq[t];
-        const int j = t - cu[s];
-        const int pos = tok_pos[t];
-        const T* sl = state + (int64_t)seq_slot[s] * state_slot_stride;
-        const float h0 = rnd<T>(x[(int64_t)t * C + c] * rinv[TAIL + i]);
-        float acc = wv[TAIL] * h0;
+        const int j = meta[i][0], pos = meta[i][1];
+        const T* sl = state + (int64_t)meta[i][2] * state_slot_stride;
+        float h0[VEC], res[VEC];
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+          h0[v] = rnd<T>(xs[i][v] * rinv[TAIL + i]);
+          res[v] = wv[v][TAIL] * h0[v];
+        }
 #pragma unroll
         for (int k = 1; k <= TAIL; ++k) {
-          float hk;
-          if (k <= j)
-            hk = win[k - 1];
-          else if (pos - k < 0)
-            hk = 0.f;
-          else
-            hk = ld(sl + (int64_t)(TAIL + j - k) * C + c);
-          acc += wv[TAIL - k] * hk;
-        }
-        st(out + (int64_t)t * C + c, h0 + acc);
 #pragma unroll
-        for (int k = TAIL; k >= 2; --k) win[k - 1] = win[k - 2];
-        if (TAIL > 0) win[0] = h0;
+          for (int v = 0; v < VEC; ++v) {
+            float hk;
+            if (k <= j)
+              hk = win[k - 1][v];
+            else if (pos - k < 0)
+              hk = 0.f;
+            else
+              hk = ld(sl + (int64_t)(TAIL + j - k) * C + c + v);
+            res[v] += wv[v][TAIL - k] * hk;
+          }
+        }
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) res[v] += h0[v];
+        st_vec<VEC>(out + (int64_t)t * C + c, res);
+#pragma unroll
+        for (int k = TAIL; k >= 2; --k)
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) win[k - 1][v] = win[k - 2][v];
+        if (TAIL > 0) {
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) win[0][v] = h0[v];
+        }
       }
     }
   }
@@ -483,19 +559,14 @@ __global__ __launch_bounds__(NT) void latent_attn_merge_k(
 typedef short bf16x8s __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-__device__ __forceinline__ short f2bf_bits(float f) {
-  union { float f; unsigned u; } c;
-  c.f = f;
-  return (short)((c.u + 0x7FFF + ((c.u >> 16) & 1)) >> 16);
-}
-
 constexpr int TB_ROWS = 128;  // rows per workgroup
 constexpr int TB_KEYS = 32;   // keys per step
 constexpr int VT_STRIDE = TB_KEYS + 8;
 
-// SPLIT = 2: two waves share a row block and each keeps half of the output
-// columns (the score product is computed twice) so that wide latents fit the
-// register file; the workgroup then owns 64 rows.
+// SPLIT = 2 (wide latents): two waves share a row block so that the operands
+// fit the register file. Each keeps half of the query's dimensions and half of
+// the output columns; the two partial score tiles are summed through LDS. The
+// workgroup then owns 64 rows.
 template <int DVB, int DKT_MAX, int SPLIT, bool PREFETCH>
 __global__ __launch_bounds__(256) void latent_attn_mfma_k(
     const short* __restrict__ q_lat,  // [H, Ttok, rank]
@@ -509,12 +580,14 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_k(
   constexpr int DVW = DVB / SPLIT;     // output blocks of this wave
   constexpr int ROWS = TB_ROWS / SPLIT;
   constexpr int CPT = (DKT_MAX + 3) / 4;  // staged 16-byte chunks per thread
+  constexpr int QKT = DKT_MAX / SPLIT;    // query fragments of this wave
   const int Dk = rank + rot;
   const int DkP = (Dk + 15) & ~15;
   const int DKT = DkP >> 4;
   const int KSS = DkP + 8;
   short* Ks = reinterpret_cast<short*>(smem_raw);  // [TB_KEYS][KSS]
   short* Vt = Ks + TB_KEYS * KSS;                  // [DVB*32][VT_STRIDE]
+  float* xch = reinterpret_cast<float*>(Vt + DVB * 32 * VT_STRIDE);  // [4][16][64]
   const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
   const int hl = lane >> 5, l31 = lane & 31;
   const int s = work[2 * blockIdx.x], m0 = work[2 * blockIdx.x + 1];
@@ -544,9 +617,12 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_k(
     return;
   }
 
-  bf16x8s qf[DKT_MAX];
+  // this wave's share of the key dimension: fragments kt_lo .. kt_lo + QKT - 1
+  const int kt_lo = part_id * QKT;
+  bf16x8s qf[QKT];
 #pragma unroll
-  for (int kt = 0; kt < DKT_MAX; ++kt) {
+  for (int i = 0; i < QKT; ++i) {
+    const int kt = kt_lo + i;
     if (kt < DKT) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
@@ -556,7 +632,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_k(
           v = q_lat[((int64_t)h * Ttok + t) * rank + d];
         else if (d < Dk)
           v = q_rot[((int64_t)t * H + h) * rot + d - rank];
-        qf[kt][e] = v;
+        qf[i][e] = v;
       }
     }
   }
@@ -634,12 +710,20 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_k(
 #pragma unroll
     for (int r = 0; r < 16; ++r) st[r] = 0.f;
 #pragma unroll
-    for (int kt = 0; kt < DKT_MAX; ++kt) {
+    for (int i = 0; i < QKT; ++i) {
+      const int kt = kt_lo + i;
       if (kt < DKT) {
         const bf16x8s kf =
             *reinterpret_cast<const bf16x8s*>(Ks + l31 * KSS + 16 * kt + 8 * hl);
-        st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kt], st, 0, 0, 0);
+        st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[i], st, 0, 0, 0);
       }
+    }
+    if (SPLIT == 2) {  // add the partner wave's half of the dot products
+#pragma unroll
+      for (int r = 0; r < 16; ++r) xch[(wid * 16 + r) * 64 + lane] = st[r];
+      __syncthreads();
+#pragma unroll
+      for (int r = 0; r < 16; ++r) st[r] += xch[((wid ^ 1) * 16 + r) * 64 + lane];
     }
     float mx = -INFINITY;
 #pragma unroll
@@ -723,7 +807,8 @@ int launch_latent_attn_mfma(const void* q_lat, const void* q_rot, const void* po
                             int Ttok, int H, int rank, int rot, int nsplit, float scale,
                             hipStream_t s) {
   const int DkP = (rank + rot + 15) & ~15;
-  const size_t lds = (size_t)TB_KEYS * (DkP + 8) * 2 + (size_t)DVB * 32 * VT_STRIDE * 2;
+  const size_t lds = (size_t)TB_KEYS * (DkP + 8) * 2 + (size_t)DVB * 32 * VT_STRIDE * 2 +
+                     (SPLIT == 2 ? 4 * 16 * 64 * 4 : 0);
   auto kern = latent_attn_mfma_k<DVB, DKT_MAX, SPLIT, PREFETCH>;
   if (lds > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -873,9 +958,14 @@ int dsv_norm_conv(const float* x, const float* gain, const void* w, void* state,
   const int tiles = (Ttok + CONV_TOKS - 1) / CONV_TOKS;
 #define TILE(N)                                                                              \
   case N:                                                                                    \
-    BY_DTYPE(dt, (norm_conv_tile_k<T, N><<<tiles, NT, 0, s>>>(                               \
-                     x, gain, (const T*)w, (const T*)state, state_slot_stride, cu, seq_slot, \
-                     tok_seq, tok_pos, (T*)out, Ttok, C, eps)));                             \
+    if (C % 4 == 0)                                                                          \
+      BY_DTYPE(dt, (norm_conv_tile_k<T, N, 4><<<tiles, NT, 0, s>>>(                          \
+                       x, gain, (const T*)w, (const T*)state, state_slot_stride, cu,         \
+                       seq_slot, tok_seq, tok_pos, (T*)out, Ttok, C, eps)));                 \
+    else                                                                                     \
+      BY_DTYPE(dt, (norm_conv_tile_k<T, N, 1><<<tiles, NT, 0, s>>>(                          \
+                       x, gain, (const T*)w, (const T*)state, state_slot_stride, cu,         \
+                       seq_slot, tok_seq, tok_pos, (T*)out, Ttok, C, eps)));                 \
     break
   switch (taps) {
     TILE(1);
@@ -961,7 +1051,7 @@ int dsv_latent_attn_mfma(const void* q_lat, const void* q_rot, const void* pool,
   if (rank <= 64 && dk <= 128) GO(2, 8, 1, true);
   if (rank <= 128 && dk <= 192) GO(4, 12, 1, true);
   if (rank <= 256 && dk <= 320) GO(8, 20, 1, true);
-  GO(16, 40, 2, false);
+  GO(16, 40, 2, true);
 #undef GO
 }
 
