@@ -252,6 +252,10 @@ class InferenceEngine(nn.Module):
 
         input_ids: [B, S] prompt. Returns [B, S + new] including the prompt.
         """
+        if hasattr(self.module, "build_cache"):
+            return self._generate_ragged(
+                input_ids, max_new_tokens, eos_token_id, do_sample=do_sample,
+                temperature=temperature, top_k=top_k, top_p=top_p)
         layers, kv_heads, head_dim, max_seq = self._model_geometry()
         if self.config.enable_cuda_graph and self.device.type == "cuda":
             from .graph import graph_generate
@@ -273,6 +277,32 @@ class InferenceEngine(nn.Module):
                            do_sample=do_sample, temperature=temperature,
                            top_k=top_k, top_p=top_p,
                            eos_token_id=eos_token_id)
+
+    def _generate_ragged(self, input_ids, max_new_tokens, eos_token_id,
+                         **sampling):
+        """generate() for models that bring their own cache manager: the prompts
+        become requests of the continuous batcher (paged state, ragged steps) and
+        run to completion together. Rows that stop early at eos are padded with
+        eos."""
+        from .ragged import ContinuousBatcher, Request
+        B, S = input_ids.shape
+        dtype = self.config.dtype if isinstance(self.config.dtype, torch.dtype) \
+            else torch.bfloat16
+        bs = 64
+        per = (S + max_new_tokens + bs - 1) // bs * bs
+        batcher = ContinuousBatcher(self.module, max_slots=B, dtype=dtype,
+                                    device=self.device, max_tokens=B * per)
+        for i in range(B):
+            batcher.put(Request(uid=i, prompt=input_ids[i].cpu().long(),
+                                max_new_tokens=max_new_tokens,
+                                eos_token_id=eos_token_id, **sampling))
+        done = {r.uid: r.generated for r in batcher.run_to_completion(
+            max_steps=4 * (S + max_new_tokens) + 16)}
+        width = max(len(g) for g in done.values())
+        pad = eos_token_id if eos_token_id is not None else 0
+        new = torch.tensor([done[i] + [pad] * (width - len(done[i]))
+                            for i in range(B)], dtype=input_ids.dtype)
+        return torch.cat([input_ids.cpu(), new], dim=1).to(input_ids.device)
 
 
 def _select_token(logits, do_sample, temperature, top_k, top_p=1.0):

@@ -121,16 +121,24 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--model", default="llama-mini",
                     choices=["llama3-8b", "llama-mini", "phi3-mini", "tiny"])
+    ap.add_argument("--model-dir", default=None,
+                    help="checkpoint folder (config.json + *.safetensors); "
+                         "config.json names the architecture")
     ap.add_argument("--port", type=int, default=8000)
     ap.add_argument("--max-slots", type=int, default=16)
     args = ap.parse_args()
-    cfg = {"llama3-8b": llama3_8b, "llama-mini": llama_mini,
-           "phi3-mini": phi3_mini, "tiny": llama_tiny}[args.model]()
-    model = LlamaForCausalLM(cfg)
     dtype = torch.bfloat16 if torch.cuda.is_available() else torch.float32
-    model = model.to(dtype)
-    if torch.cuda.is_available():
-        model = model.cuda()
+    if args.model_dir:
+        from ..models import load_pretrained
+        model = load_pretrained(
+            args.model_dir, dtype=dtype,
+            device="cuda" if torch.cuda.is_available() else "cpu")
+    else:
+        cfg = {"llama3-8b": llama3_8b, "llama-mini": llama_mini,
+               "phi3-mini": phi3_mini, "tiny": llama_tiny}[args.model]()
+        model = LlamaForCausalLM(cfg).to(dtype)
+        if torch.cuda.is_available():
+            model = model.cuda()
     server = InferenceServer(model, max_slots=args.max_slots,
                              dtype=dtype).start()
     uvicorn.run(build_app(server), host="127.0.0.1", port=args.port)

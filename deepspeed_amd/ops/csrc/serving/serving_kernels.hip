@@ -562,6 +562,7 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 constexpr int TB_ROWS = 128;  // rows per workgroup
 constexpr int TB_KEYS = 32;   // keys per step
 constexpr int VT_STRIDE = TB_KEYS + 8;
+constexpr float LAZY_MAX = 8.f;
 
 // SPLIT = 2 (wide latents): two waves share a row block so that the operands
 // fit the register file. Each keeps half of the query's dimensions and half of
@@ -619,20 +620,28 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_k(
 
   // this wave's share of the key dimension: fragments kt_lo .. kt_lo + QKT - 1
   const int kt_lo = part_id * QKT;
+  const bool q_vec = (rank & 7) == 0 && (rot & 7) == 0;
   bf16x8s qf[QKT];
 #pragma unroll
   for (int i = 0; i < QKT; ++i) {
     const int kt = kt_lo + i;
     if (kt < DKT) {
+      const int d0 = 16 * kt + 8 * hl;
+      if (q_vec && d0 + 8 <= rank) {
+        qf[i] = *reinterpret_cast<const bf16x8s*>(q_lat + ((int64_t)h * Ttok + t) * rank + d0);
+      } else if (q_vec && d0 >= rank && d0 + 8 <= Dk) {
+        qf[i] = *reinterpret_cast<const bf16x8s*>(q_rot + ((int64_t)t * H + h) * rot + d0 - rank);
+      } else {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int d = 16 * kt + 8 * hl + e;
-        short v = 0;
-        if (d < rank)
-          v = q_lat[((int64_t)h * Ttok + t) * rank + d];
-        else if (d < Dk)
-          v = q_rot[((int64_t)t * H + h) * rot + d - rank];
-        qf[i][e] = v;
+        for (int e = 0; e < 8; ++e) {
+          const int d = d0 + e;
+          short v = 0;
+          if (d < rank)
+            v = q_lat[((int64_t)h * Ttok + t) * rank + d];
+          else if (d < Dk)
+            v = q_rot[((int64_t)t * H + h) * rot + d - rank];
+          qf[i][e] = v;
+        }
       }
     }
   }
@@ -692,8 +701,16 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_k(
 #pragma unroll
       for (int i = 0; i < CPT; ++i) stash_one(i, pre[i]);
     } else {
+      // a few loads in flight at a time: enough to overlap their latency,
+      // few enough to stay in registers
 #pragma unroll 1
-      for (int i = 0; i < CPT; ++i) stash_one(i, fetch_one(i, k0));
+      for (int i = 0; i < CPT; i += 5) {
+        bf16x8s v[5];
+#pragma unroll
+        for (int u = 0; u < 5; ++u) v[u] = fetch_one(i + u, k0);
+#pragma unroll
+        for (int u = 0; u < 5; ++u) stash_one(i + u, v[u]);
+      }
     }
   };
 
@@ -734,25 +751,30 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_k(
       mx = fmaxf(mx, v);
     }
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float m_new = fmaxf(mrun, mx);
-    // a row that has seen no key yet (a later split of an early token) keeps
-    // weight zero without producing inf - inf
+    // The running maximum follows the scores lazily: it moves only when a
+    // score exceeds it by more than LAZY_MAX (weights stay below e^LAZY_MAX,
+    // harmless in fp32), so most steps need no rescaling of the sums at all.
+    // A row that has seen no key yet (a later split of an early token) keeps
+    // weight zero without producing inf - inf.
+    const float m_new = (mx > mrun + LAZY_MAX) ? mx : mrun;
     const float m_use = m_new == -INFINITY ? 0.f : m_new;
-    const float alpha = expf(mrun - m_use);
+    const float alpha = __expf(mrun - m_use);
     float psum = 0.f;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      const float p = expf(st[r] - m_use);
+      const float p = __expf(st[r] - m_use);
       st[r] = p;
       psum += p;
     }
     psum += __shfl_xor(psum, 32, 64);
     lrun = lrun * alpha + psum;
+    if (__any(m_new != mrun)) {
+#pragma unroll
+      for (int db = 0; db < DVW; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
+    }
     mrun = m_new;
-#pragma unroll
-    for (int db = 0; db < DVW; ++db)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
       // B fragment of P: keys 16*ks + 8*hl + 0..7 of this lane's row; half of
@@ -1051,7 +1073,7 @@ int dsv_latent_attn_mfma(const void* q_lat, const void* q_rot, const void* pool,
   if (rank <= 64 && dk <= 128) GO(2, 8, 1, true);
   if (rank <= 128 && dk <= 192) GO(4, 12, 1, true);
   if (rank <= 256 && dk <= 320) GO(8, 20, 1, true);
-  GO(16, 40, 2, true);
+  GO(16, 40, 2, false);
 #undef GO
 }
 

@@ -41,7 +41,8 @@ ext = CUDAExtension(
     ],
     extra_compile_args={
         "cxx": ["-O3", "-std=c++17", "-fopenmp", "-mavx2", "-mfma"],
-        "nvcc": ["-O3", "-std=c++17", "--offload-arch=gfx950"],
+        "nvcc": ["-O3", "-std=c++17", "--offload-arch=gfx950",
+                 "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"],
     },
     extra_link_args=["-fopenmp"],
 )
