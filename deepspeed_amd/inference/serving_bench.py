@@ -163,11 +163,19 @@ def _kernel_rows(z, dev):
     cw = torch.randn(W, 4, device=dev).to(bf)
     wn = torch.ones(W, device=dev, dtype=bf)
     batch = cache.begin_ragged(list(range(B)), [S] * B)
+    delta = torch.randn(T, W, device=dev).to(bf) * 0.01
+    ssq = sk.residual_add_stats(x32, delta)
     row("norm_conv (fp32 stream in, bf16 out, 4 taps)", "rms_norm",
         lambda: sk.norm_conv_ragged(x32, gain, 1e-6, cw,
-                                    cache.states["conv"][:, 0], batch, bf),
+                                    cache.states["conv"][:, 0], batch, bf,
+                                    ssq),
         T * W * 6)
     row("rms_norm (llama)", "", lambda: rms_norm(x16, wn, 1e-6), T * W * 4)
+    row("residual_add_stats (fp32 stream += bf16, row sums)", "add",
+        lambda: sk.residual_add_stats(x32, delta), T * W * 10)
+    y16 = torch.empty_like(x16)
+    row("add (llama residual, bf16)", "",
+        lambda: torch.add(x16, delta, out=y16), T * W * 6)
     # ---- prefill attention
     q_lat = (torch.randn(H, T, rank, device=dev) * 0.1).to(bf)
     q_rot = (torch.randn(T, H, rot, device=dev) * 0.1).to(bf)

@@ -27,7 +27,7 @@ import torch.nn.functional as F
 from ..inference.state_cache import PagedStateCache
 from ..moe.routed import RoutedExperts
 from ..ops.activations import xielu
-from ..ops.causal_conv import norm_conv_ragged
+from ..ops.causal_conv import norm_conv_ragged, residual_add_stats
 from ..ops.latent_attention import (gate_merge_heads, latent_attention,
                                     latent_prep)
 from ..ops.norms import ScalarRMSNorm
@@ -160,18 +160,22 @@ class FizesunLayer(nn.Module):
             else:
                 raise ValueError(f"unknown mlp kind {mlp['kind']!r}")
 
-    def forward(self, x, cache, stream, dtype, max_pos):
+    def forward(self, x, cache, stream, dtype, max_pos, sumsq=None):
+        """x: fp32 stream, updated in place. ``sumsq``: row sums of squares of
+        x when its producer computed them. Returns the sums of the new x (or
+        None) for the next layer's first norm."""
         b = cache.batch
         h = norm_conv_ragged(x, self.norm1.gain, self.norm1.eps, self.conv1,
-                             cache.states["conv"][:, 2 * stream], b, dtype)
-        x = x.add_(self.mixer(h, cache, stream, max_pos))
+                             cache.states["conv"][:, 2 * stream], b, dtype,
+                             sumsq)
+        sumsq = residual_add_stats(x, self.mixer(h, cache, stream, max_pos))
         if self.mlp is not None:
             h = norm_conv_ragged(x, self.norm2.gain, self.norm2.eps,
                                  self.conv2,
                                  cache.states["conv"][:, 2 * stream + 1], b,
-                                 dtype)
-            x = x.add_(self.mlp(h))
-        return x
+                                 dtype, sumsq)
+            sumsq = residual_add_stats(x, self.mlp(h))
+        return sumsq
 
 
 class FizesunForCausalLM(nn.Module):
@@ -297,11 +301,13 @@ class FizesunForCausalLM(nn.Module):
         max_pos = cache.max_seq
         x0 = self.embed_norm(self.embed, out_dtype=torch.float32, index=ids)
         x = x0.clone()
+        sumsq = None
         for stream, (i, t, enters) in enumerate(self.runs):
             if enters:
                 x = F.linear(torch.cat([x, x0], -1).to(dt), self.loop_in) \
                     .float().add_(self.loop_step[t])
-            x = self.layers[i](x, cache, stream, dt, max_pos)
+                sumsq = None
+            sumsq = self.layers[i](x, cache, stream, dt, max_pos, sumsq)
             if taps is not None:
                 taps.append(x.clone())
         return F.linear(self.final_norm(x, out_dtype=dt, index=rows),

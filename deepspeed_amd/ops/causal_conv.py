@@ -26,14 +26,16 @@ def _norm(x, gain, eps, dtype):
             * gain.float().reshape(())).to(dtype)
 
 
-def norm_conv_ragged(x, gain, eps, conv_w, state, batch, out_dtype):
+def norm_conv_ragged(x, gain, eps, conv_w, state, batch, out_dtype,
+                     sumsq=None):
     """x [T, C] fp32 residual; conv_w [C, taps]; state [slots, taps-1, C]
     (updated in place); batch: RaggedBatch. Returns h + conv(h) as
-    [T, C] ``out_dtype``."""
+    [T, C] ``out_dtype``. ``sumsq`` ([T] fp32, from ``residual_add_stats``)
+    spares the kernel its own reduction over x."""
     if x.is_cuda and _sk().enabled():
         sk = _sk()
         return sk.norm_conv_ragged(x, gain, eps, conv_w, state, batch,
-                                   out_dtype)
+                                   out_dtype, sumsq)
     taps = conv_w.shape[1]
     h = _norm(x, gain, eps, out_dtype)
     out = torch.empty_like(h)
@@ -48,3 +50,13 @@ def norm_conv_ragged(x, gain, eps, conv_w, state, batch, out_dtype):
             state[slot] = hist[-(taps - 1):].to(state.dtype)
         at += count
     return out
+
+
+def residual_add_stats(x, delta):
+    """x += delta (fp32 stream, delta in the compute dtype), in place. On the
+    GPU the same pass returns every row's sum of squares for the norm that
+    follows; the eager path returns None and the norm reduces by itself."""
+    if x.is_cuda and _sk().enabled():
+        return _sk().residual_add_stats(x, delta)
+    x.add_(delta)
+    return None

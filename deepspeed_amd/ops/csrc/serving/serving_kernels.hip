@@ -170,8 +170,9 @@ __global__ __launch_bounds__(NT) void norm_conv_tile_k(
     const T* __restrict__ w, const T* __restrict__ state,
     int64_t state_slot_stride, const int* __restrict__ cu,
     const int* __restrict__ seq_slot, const int* __restrict__ tok_seq,
-    const int* __restrict__ tok_pos, T* __restrict__ out, int Ttok, int C,
-    float eps) {
+    const int* __restrict__ tok_pos, T* __restrict__ out,
+    const float* __restrict__ sumsq,  // optional: sum of x^2 per row
+    int Ttok, int C, float eps) {
   constexpr int TAIL = TAPS - 1;
   constexpr int NR = CONV_TOKS + TAIL;
   __shared__ float rinv[NR];
@@ -185,6 +186,13 @@ __global__ __launch_bounds__(NT) void norm_conv_tile_k(
     meta[threadIdx.x][1] = tok_pos[t];
     meta[threadIdx.x][2] = seq_slot[s];
   }
+  if (sumsq) {  // the producer of x already summed its squares
+    if (threadIdx.x < NR) {
+      const int tt = t0 - TAIL + threadIdx.x;
+      const float ss = (tt >= 0 && tt < Ttok) ? sumsq[tt] : 0.f;
+      rinv[threadIdx.x] = rsqrtf(ss / (float)C + eps) * g;
+    }
+  } else
   for (int ri = wid; ri < NR; ri += NT / 64) {
     const int tt = t0 - TAIL + ri;
     float ss = 0.f;
@@ -265,6 +273,31 @@ __global__ __launch_bounds__(NT) void norm_conv_tile_k(
       }
     }
   }
+}
+
+// x += delta (fp32 stream, delta in the compute type) and the sum of squares
+// of every updated row, which the next norm needs: the norm's reduction rides
+// on the pass that has to touch the stream anyway.
+template <typename T, int VEC>
+__global__ __launch_bounds__(NT) void residual_add_stats_k(
+    float* __restrict__ x, const T* __restrict__ delta, float* __restrict__ sumsq, int C) {
+  __shared__ float red[NT / 64];
+  const int64_t r = blockIdx.x;
+  float* row = x + r * C;
+  const T* drow = delta + r * C;
+  float ss = 0.f;
+  for (int c = threadIdx.x * VEC; c < C; c += NT * VEC) {
+    float v[VEC];
+    ld_vec<VEC>(row + c, v);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      v[i] += ld(drow + c + i);
+      ss += v[i] * v[i];
+    }
+    st_vec<VEC>(row + c, v);
+  }
+  ss = block_sum(ss, red);
+  if (threadIdx.x == 0) sumsq[r] = ss;
 }
 
 // One block per sequence: the tail becomes the last taps-1 normed inputs.
@@ -974,7 +1007,8 @@ int dsv_scalar_rms_norm(const void* x, int in_dt, const int64_t* idx, const floa
 int dsv_norm_conv(const float* x, const float* gain, const void* w, void* state,
                   int64_t state_slot_stride, const int* cu, const int* seq_slot,
                   const int* seq_start, const int* tok_seq, const int* tok_pos, void* out,
-                  int dt, int Ttok, int nseq, int C, int taps, float eps, hipStream_t s) {
+                  const float* sumsq, int dt, int Ttok, int nseq, int C, int taps, float eps,
+                  hipStream_t s) {
   if (taps > MAXTAPS) return -1;
   if (Ttok <= 0) return 0;
   const int tiles = (Ttok + CONV_TOKS - 1) / CONV_TOKS;
@@ -983,11 +1017,11 @@ int dsv_norm_conv(const float* x, const float* gain, const void* w, void* state,
     if (C % 4 == 0)                                                                          \
       BY_DTYPE(dt, (norm_conv_tile_k<T, N, 4><<<tiles, NT, 0, s>>>(                          \
                        x, gain, (const T*)w, (const T*)state, state_slot_stride, cu,         \
-                       seq_slot, tok_seq, tok_pos, (T*)out, Ttok, C, eps)));                 \
+                       seq_slot, tok_seq, tok_pos, (T*)out, sumsq, Ttok, C, eps)));          \
     else                                                                                     \
       BY_DTYPE(dt, (norm_conv_tile_k<T, N, 1><<<tiles, NT, 0, s>>>(                          \
                        x, gain, (const T*)w, (const T*)state, state_slot_stride, cu,         \
-                       seq_slot, tok_seq, tok_pos, (T*)out, Ttok, C, eps)));                 \
+                       seq_slot, tok_seq, tok_pos, (T*)out, sumsq, Ttok, C, eps)));          \
     break
   switch (taps) {
     TILE(1);
@@ -1008,6 +1042,16 @@ int dsv_norm_conv(const float* x, const float* gain, const void* w, void* state,
   if (taps > 1)
     BY_DTYPE(dt, (conv_tail_k<T><<<nseq, NT, 0, s>>>(x, gain, (T*)state, state_slot_stride, cu,
                                                       seq_slot, seq_start, C, taps, eps)));
+  return (int)hipGetLastError();
+}
+
+int dsv_residual_add_stats(float* x, const void* delta, float* sumsq, int dt, int rows, int C,
+                           hipStream_t s) {
+  if (rows <= 0) return 0;
+  if (C % 4 == 0)
+    BY_DTYPE(dt, (residual_add_stats_k<T, 4><<<rows, NT, 0, s>>>(x, (const T*)delta, sumsq, C)));
+  else
+    BY_DTYPE(dt, (residual_add_stats_k<T, 1><<<rows, NT, 0, s>>>(x, (const T*)delta, sumsq, C)));
   return (int)hipGetLastError();
 }
 

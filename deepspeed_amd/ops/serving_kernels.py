@@ -118,7 +118,8 @@ def scalar_rms_norm(x, gain, eps, out_dtype, index=None):
     return out
 
 
-def norm_conv_ragged(x, gain, eps, conv_w, state, batch, out_dtype):
+def norm_conv_ragged(x, gain, eps, conv_w, state, batch, out_dtype,
+                     sumsq=None):
     T, C = x.shape
     taps = conv_w.shape[1]
     assert x.dtype == torch.float32 and x.is_contiguous()
@@ -127,15 +128,30 @@ def norm_conv_ragged(x, gain, eps, conv_w, state, batch, out_dtype):
     assert state.shape[1:] == (taps - 1, C)
     assert state.stride(2) == 1 and (taps == 1 or state.stride(1) == C)
     assert T == batch.n_tokens
+    assert sumsq is None or (sumsq.dtype == torch.float32
+                             and sumsq.numel() == T)
     out = torch.empty(T, C, dtype=out_dtype, device=x.device)
     _check(load().dsv_norm_conv(
         _p(x), _p(_f32(gain).reshape(1)), _p(conv_w),
         ctypes.c_void_p(state.data_ptr()), _l(state.stride(0)),
         _p(batch.cu), _p(batch.seq_slot), _p(batch.seq_start),
-        _p(batch.tok_seq), _p(batch.tok_pos), _p(out), _i(_DT[out_dtype]),
-        _i(T), _i(batch.n_seqs), _i(C), _i(taps), _f(eps), _stream()),
+        _p(batch.tok_seq), _p(batch.tok_pos), _p(out), _p(sumsq),
+        _i(_DT[out_dtype]), _i(T), _i(batch.n_seqs), _i(C), _i(taps), _f(eps), _stream()),
         "norm_conv")
     return out
+
+
+def residual_add_stats(x, delta):
+    """x += delta in place; returns the per-row sums of squares of the new x."""
+    T, C = x.shape
+    assert x.dtype == torch.float32 and x.is_contiguous()
+    assert delta.shape == x.shape
+    delta = delta.contiguous()
+    sumsq = torch.empty(T, dtype=torch.float32, device=x.device)
+    _check(load().dsv_residual_add_stats(_p(x), _p(delta), _p(sumsq),
+                                         _i(_dt(delta)), _i(T), _i(C),
+                                         _stream()), "residual_add_stats")
+    return sumsq
 
 
 # ------------------------------------------------------ latent attention
