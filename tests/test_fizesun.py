@@ -456,6 +456,51 @@ def test_bfloat16_stays_near_the_oracle():
     close_rms(s.run(t, [7, 1, 20, 1, 1]), want, 0.06)
 
 
+# ---------------------------------------------- mid size, default 64-token blocks
+def _mid_config(top):
+    a = mixer(heads=5, dim=24, rot_dim=12, vdim=20, rank=40, dims=8, base=3000.0)
+    b = mixer(heads=2, dim=32, rot_dim=8, vdim=32, rank=24, base=700.0)
+    return config([(a, moe(6, top, ff=28, limit=1.2, shared=False)),
+                   (b, dense(150)), (a, moe(6, top, ff=36, limit=3.0))],
+                  width=96, vocab=131, taps=5, loop=(0, 2, 2), eps=1e-6)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_mid_size_mixed_schedule_over_block_borders(dtype):
+    """Three requests of 150, 70 and 5 tokens share steps: portions that end
+    on and off the 64-token block borders beside single tokens; five layer
+    runs with two attention shapes."""
+    cfg = _mid_config(3 if dtype == torch.float32 else 6)
+    s = Served(cfg, seed=21, dtype=dtype, slots=3, max_tokens=64 * 6, block=64)
+    seqs = {"a": toks(150, 131, seed=31), "b": toks(70, 131, seed=32),
+            "c": toks(5, 131, seed=33)}
+    steps = [{"a": 67, "b": 2}, {"a": 61, "b": 62, "c": 5}, {"a": 1, "b": 1},
+             {"a": 1, "b": 1}, {"b": 4, "a": 2}, {"a": 18}]
+    reqs, at, got = {}, {k: 0 for k in seqs}, {k: [] for k in seqs}
+    for step in steps:
+        entries = []
+        for k, n in step.items():
+            if k not in reqs:
+                reqs[k] = s.batcher.open(k)
+            entries.append((reqs[k], seqs[k][at[k]:at[k] + n]))
+        out = s.batcher.feed(entries).double().cpu()
+        o = 0
+        for k, n in step.items():
+            got[k].append(out[o:o + n])
+            o += n
+            at[k] += n
+            if at[k] == len(seqs[k]):
+                s.batcher.close(reqs[k])
+    for k, t in seqs.items():
+        assert at[k] == len(t)
+        if dtype == torch.float32:
+            close(torch.cat(got[k]), s.oracle(t), 3e-4)
+        else:
+            # five layer runs of unit-gain random weights amplify 16-bit
+            # rounding; the sharp comparison is the 32-bit one above
+            close_rms(torch.cat(got[k]), s.oracle(t), 0.15)
+
+
 # -------------------------------------------- the framework's entry points
 def test_greedy_generation_through_the_scheduler(base):
     prompts = [toks(n, seed=60 + n) for n in (3, 12, 18)]
