@@ -53,6 +53,8 @@ def main(argv=None):
         for e in step["entries"]:
             if e["id"] not in live:
                 live[e["id"]] = batcher.open(e["id"])
+            if not e["tokens"]:
+                continue                 # admitted, nothing to run yet
             entries.append((live[e["id"]], e["tokens"]))
             rows += [at + w for w in e.get("want", [])]
             at += len(e["tokens"])

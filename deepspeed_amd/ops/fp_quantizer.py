@@ -81,7 +81,10 @@ def fp_dequantize(q: torch.Tensor, scales: torch.Tensor, numel: int,
                   out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
     from ._loader import get_ext
     ext = get_ext()
-    return ext.fp_dequantize(q, scales, numel, group_size, bits, out_dtype)
+    # group scales are fp32 in the kernel; a module-wide .to(bf16) may have
+    # narrowed the buffer that holds them
+    return ext.fp_dequantize(q, scales.float(), numel, group_size, bits,
+                             out_dtype)
 
 
 def fp_emulate_reference(x: torch.Tensor, bits: int = 6,
