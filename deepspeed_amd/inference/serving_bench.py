@@ -212,6 +212,31 @@ def _kernel_rows(z, dev):
     row("paged_decode (llama)", "",
         lambda: paged_decode_attention(qd, kp, kp, table, lens),
         B * (S + 1) * hkv * 128 * 2 * 2)
+    # ---- the same at 64 requests, where the bytes of the cache matter
+    NB = 64
+    big = PagedStateCache([rank + rot], {}, NB, NB * (S + 64), dtype=bf,
+                          device=dev)
+    big.pools[0].normal_()
+    for i in range(NB):
+        big.lens[i] = S
+    batch = big.begin_ragged(list(range(NB)), [1] * NB)
+    qb_lat = (torch.randn(H, NB, rank, device=dev) * 0.1).to(bf)
+    qb_rot = (torch.randn(NB, H, rot, device=dev) * 0.1).to(bf)
+    row("latent_attention decode, 64 requests", "paged_decode",
+        lambda: sk.latent_attention(qb_lat, qb_rot, big.pools[0], batch, rank,
+                                    0.07),
+        NB * (S + 1) * (rank + rot) * 2)
+    big.end_step()
+    del big
+    nb = NB * ((S + 64) // 64)
+    kp = torch.randn(nb, hkv, 64, 128, device=dev).to(bf)
+    table = torch.arange(nb, dtype=torch.int32, device=dev).view(NB, -1)
+    lens = torch.full((NB,), S + 1, dtype=torch.int32, device=dev)
+    qd = torch.randn(NB, H, 128, device=dev).to(bf)
+    row("paged_decode, 64 requests (llama)", "",
+        lambda: paged_decode_attention(qd, kp, kp, table, lens),
+        NB * (S + 1) * hkv * 128 * 2 * 2)
+    del kp
     # ---- activations
     zf = torch.randn(T, F, device=dev).to(bf)
     pq = torch.zeros(2, device=dev)
