@@ -29,29 +29,45 @@ HIPCC_FLAGS = ["-O3", "-std=c++17", "--offload-arch=gfx950",
 _lib = None
 
 
-def build(force=True):
-    """Compile the library in-tree (cross-compiles without a GPU)."""
-    if not force and os.path.exists(LIBRARY) and \
-            os.path.getmtime(LIBRARY) >= os.path.getmtime(SOURCE):
-        return LIBRARY
+def _compile(target):
     hipcc = os.environ.get("HIPCC") or (
         "/opt/rocm/bin/hipcc" if os.path.exists("/opt/rocm/bin/hipcc")
         else "hipcc")
-    tmp = "%s.%d.tmp" % (LIBRARY, os.getpid())
+    tmp = "%s.%d.tmp" % (target, os.getpid())
     cmd = [hipcc] + HIPCC_FLAGS + ["-o", tmp, SOURCE]
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
                        text=True)
     if r.returncode != 0:
         raise RuntimeError("building the serving kernels failed:\n" + r.stdout)
-    os.replace(tmp, LIBRARY)
-    return LIBRARY
+    os.replace(tmp, target)
+    return target
+
+
+def _fresh(path):
+    return os.path.exists(path) and \
+        os.path.getmtime(path) >= os.path.getmtime(SOURCE)
+
+
+def build(force=True):
+    """Compile the library in-tree (cross-compiles without a GPU). Returns the
+    path of the library to load. Where the tree cannot be written, a copy
+    keyed by the source's content goes to the temporary directory instead."""
+    if not force and _fresh(LIBRARY):
+        return LIBRARY
+    if os.access(os.path.dirname(LIBRARY), os.W_OK):
+        return _compile(LIBRARY)
+    import hashlib
+    import tempfile
+    with open(SOURCE, "rb") as f:
+        tag = hashlib.sha1(f.read()).hexdigest()[:16]
+    alt = os.path.join(tempfile.gettempdir(), "ds_amd_serving_%s.so" % tag)
+    return alt if os.path.exists(alt) else _compile(alt)
 
 
 def load():
     global _lib
     if _lib is None:
-        build(force=False)
-        _lib = ctypes.CDLL(LIBRARY)
+        _lib = ctypes.CDLL(build(force=False))
         _lib.dsv_latent_attn_lds.restype = ctypes.c_int64
     return _lib
 

@@ -581,6 +581,34 @@ def test_schedule_replay_runner(tmp_path):
         close(torch.from_numpy(got).double(), ref)
 
 
+def test_generate_command_line(tmp_path):
+    """bin/ds_generate: registry -> init_inference -> generate, greedy."""
+    import subprocess
+    import sys
+    from safetensors.torch import save_file
+    cfg = VARIANTS["no_loop"]
+    t = tensors(cfg, seed=14)
+    (tmp_path / "config.json").write_text(json.dumps(cfg))
+    save_file({k: v.bfloat16().contiguous() for k, v in t.items()},
+              str(tmp_path / "model.safetensors"))
+    a, b = toks(6, seed=70), toks(6, seed=71)
+    repo = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    p = subprocess.run(
+        [sys.executable, os.path.join(repo, "bin", "ds_generate"),
+         "--model-dir", str(tmp_path), "--dtype", "float32", "--max-new-tokens",
+         "3", "--tokens", ",".join(map(str, a)), "--tokens",
+         ",".join(map(str, b))], text=True, capture_output=True, timeout=600)
+    assert p.returncode == 0, p.stderr[-2000:]
+    lines = [json.loads(l) for l in p.stdout.split("\n")
+             if l.startswith("{")]
+    w = {k: v.double() for k, v in t.items()}
+    for prompt, line in zip((a, b), lines):
+        seq = list(prompt)
+        for _ in range(3):
+            seq.append(int(O.forward(cfg, w, seq)[-1].argmax()))
+        assert line["generated"] == seq[len(prompt):]
+
+
 # ------------------------------------------- HIP kernels against eager ops
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
