@@ -689,24 +689,27 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_k(
 
   // Staging: chunk c of a tile is (dims 8*(c>>5).., key c&31): neighbouring
   // lanes take neighbouring keys, so the transposed writes fall into one row.
-  auto fetch_one = [&](int i, int k0) -> bf16x8s {
+  // Every chunk of a thread belongs to the same key (256 is a multiple of 32),
+  // so the thread resolves ONE pool row per tile through the block table, and
+  // does so a step ahead: the data loads never wait for a table load.
+  auto row_of = [&](int k0) -> int64_t {
+    const int p = k0 + (tid & 31);
+    return p <= kmax ? (int64_t)tab[p / bs] * bs + p % bs : (int64_t)-1;
+  };
+  auto fetch_one = [&](int i, int64_t row) -> bf16x8s {
     const int c = tid + i * 256;
     bf16x8s v;
 #pragma unroll
     for (int e = 0; e < 8; ++e) v[e] = 0;
-    if (c < TB_KEYS * cpk) {
-      const int ch = c >> 5, key = c & 31;
-      const int p = k0 + key;
-      if (p <= kmax) {
-        const int64_t row = (int64_t)tab[p / bs] * bs + p % bs;
-        const short* src = pool + row * Dk + ch * 8;
-        if (vec_ok && ch * 8 + 8 <= Dk) {
-          v = *reinterpret_cast<const bf16x8s*>(src);
-        } else {
+    if (c < TB_KEYS * cpk && row >= 0) {
+      const int ch = c >> 5;
+      const short* src = pool + row * Dk + ch * 8;
+      if (vec_ok && ch * 8 + 8 <= Dk) {
+        v = *reinterpret_cast<const bf16x8s*>(src);
+      } else {
 #pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (ch * 8 + e < Dk) v[e] = src[e];
-        }
+        for (int e = 0; e < 8; ++e)
+          if (ch * 8 + e < Dk) v[e] = src[e];
       }
     }
     return v;
@@ -724,38 +727,48 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_k(
     }
   };
   bf16x8s pre[PREFETCH ? CPT : 1];
-  auto fetch = [&](int k0) {
+  auto fetch = [&](int64_t row) {
 #pragma unroll
     for (int i = 0; i < CPT; ++i)
-      if (PREFETCH) pre[i] = fetch_one(i, k0);
+      if (PREFETCH) pre[i] = fetch_one(i, row);
   };
-  auto stash = [&](int k0) {
+  auto stash = [&](int64_t row) {
     if (PREFETCH) {
 #pragma unroll
       for (int i = 0; i < CPT; ++i) stash_one(i, pre[i]);
     } else {
-      // a few loads in flight at a time: enough to overlap their latency,
-      // few enough to stay in registers
+      // the tile's loads all in flight, consumed before the products start
+      // (registers that live only here, unlike a prefetch across the step)
 #pragma unroll 1
-      for (int i = 0; i < CPT; i += 5) {
-        bf16x8s v[5];
+      for (int i = 0; i < CPT; i += 10) {
+        bf16x8s v[10];
 #pragma unroll
-        for (int u = 0; u < 5; ++u) v[u] = fetch_one(i + u, k0);
+        for (int u = 0; u < 10; ++u) v[u] = fetch_one(i + u, row);
 #pragma unroll
-        for (int u = 0; u < 5; ++u) stash_one(i + u, v[u]);
+        for (int u = 0; u < 10; ++u) stash_one(i + u, v[u]);
       }
     }
   };
 
   // PREFETCH keeps the next tile's loads in flight during the products; the
-  // widest class has no registers to spare for that
-  if (PREFETCH) fetch(s_lo * TB_KEYS);
+  // widest class has no registers to spare for that. row_next is the pool
+  // row of this thread's key in the tile that is fetched next.
+  int64_t row_next = row_of(s_lo * TB_KEYS);
+  if (PREFETCH) {
+    fetch(row_next);
+    row_next = row_of((s_lo + 1) * TB_KEYS);
+  }
   for (int step = s_lo; step < s_hi; ++step) {
     const int k0 = step * TB_KEYS;
     __syncthreads();
-    stash(k0);
+    stash(row_next);          // without PREFETCH: fetches tile `step` itself
     __syncthreads();
-    if (PREFETCH && step + 1 < s_hi) fetch(k0 + TB_KEYS);
+    if (PREFETCH) {
+      if (step + 1 < s_hi) fetch(row_next);
+      row_next = row_of(k0 + 2 * TB_KEYS);
+    } else {
+      row_next = row_of(k0 + TB_KEYS);
+    }
     f32x16 st;
 #pragma unroll
     for (int r = 0; r < 16; ++r) st[r] = 0.f;
