@@ -306,7 +306,8 @@ __global__ __launch_bounds__(NT) void conv_tail_k(
     const float* __restrict__ x, const float* __restrict__ gain,
     T* __restrict__ state, int64_t state_slot_stride,
     const int* __restrict__ cu, const int* __restrict__ seq_slot,
-    const int* __restrict__ seq_start, int C, int taps, float eps) {
+    const int* __restrict__ seq_start, const float* __restrict__ sumsq, int C, int taps,
+    float eps) {
   __shared__ float red[NT / 64];
   const int s = blockIdx.x;
   const int tail = taps - 1;
@@ -319,10 +320,15 @@ __global__ __launch_bounds__(NT) void conv_tail_k(
     scale[i] = 0.f;
     const int p = start + count - tail + i;  // absolute position kept at i
     if (p >= start) {
-      const float* row = x + (int64_t)(cu[s] + p - start) * C;
-      float ss = 0.f;
-      for (int c = threadIdx.x; c < C; c += NT) ss += row[c] * row[c];
-      ss = block_sum(ss, red);
+      float ss;
+      if (sumsq) {
+        ss = sumsq[cu[s] + p - start];
+      } else {
+        const float* row = x + (int64_t)(cu[s] + p - start) * C;
+        ss = 0.f;
+        for (int c = threadIdx.x; c < C; c += NT) ss += row[c] * row[c];
+        ss = block_sum(ss, red);
+      }
       scale[i] = rsqrtf(ss / (float)C + eps) * g;
     }
   }
@@ -1054,7 +1060,7 @@ int dsv_norm_conv(const float* x, const float* gain, const void* w, void* state,
 #undef TILE
   if (taps > 1)
     BY_DTYPE(dt, (conv_tail_k<T><<<nseq, NT, 0, s>>>(x, gain, (T*)state, state_slot_stride, cu,
-                                                      seq_slot, seq_start, C, taps, eps)));
+                                                      seq_slot, seq_start, sumsq, C, taps, eps)));
   return (int)hipGetLastError();
 }
 
