@@ -676,3 +676,35 @@ def test_mfma_tiles_match_the_exact_kernel(heads, rank, rot):
     # the weights are rounded to 16 bits before the second product
     assert (a - e).abs().max().item() < 0.03
     assert ((a - e) ** 2).mean().sqrt().item() < 0.004
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_exact_kernel_with_more_heads_than_one_group(dtype, monkeypatch):
+    """11 heads (the exact kernel walks heads in groups of 8), with and
+    without key splits, against the eager formulation."""
+    from deepspeed_amd.ops import latent_attention as la
+    from deepspeed_amd.ops import serving_kernels as sk
+    heads, rank, rot, bs = 11, 40, 8, 16
+    g = torch.Generator().manual_seed(5)
+    cache = PagedStateCache([rank + rot], {}, 3, 2048, block_size=bs,
+                            dtype=dtype, device=DEV)
+    for held, counts in (([0, 200, 37], [90, 1, 30]), ([700, 650], [1, 2])):
+        for slot in range(3):
+            cache.reset_slot(slot)
+        for slot, n in enumerate(held):
+            cache.lens[slot] = n
+        b = cache.begin_ragged(list(range(len(held))), counts)
+        cache.pools[0].copy_(torch.randn(cache.pools[0].shape, generator=g))
+        T = sum(counts)
+        q_lat = (torch.randn(heads, T, rank, generator=g) * 0.3).to(DEV, dtype)
+        q_rot = torch.randn(T, heads, rot, generator=g).to(DEV, dtype)
+        got = sk.latent_attention(q_lat, q_rot, cache.pools[0], b, rank, 0.2,
+                                  path="exact").float().cpu()
+        monkeypatch.setenv("DS_AMD_SERVING_EAGER", "1")
+        want = la.latent_attention(q_lat, q_rot, cache.pools[0], b, rank,
+                                   0.2).float().cpu()
+        monkeypatch.delenv("DS_AMD_SERVING_EAGER")
+        cache.end_step()
+        tol = 2e-5 if dtype == torch.float32 else 2e-2
+        assert (got - want).abs().max().item() < tol
