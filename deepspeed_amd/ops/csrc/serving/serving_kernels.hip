@@ -78,7 +78,7 @@ __global__ __launch_bounds__(NT) void scalar_rms_norm_k(
 }
 
 // ------------------------------------------------- norm + causal conv
-constexpr int MAXTAPS = 16;
+constexpr int MAXTAPS = 32;
 
 // One block per token. h = round_T(norm(x)); out = h_t + sum_k w[c][taps-1-k]
 // * h_(t-k). Earlier inputs come from this step's rows when the sequence
