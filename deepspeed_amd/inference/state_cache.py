@@ -62,7 +62,9 @@ class PagedStateCache:
                  num_slots: int, max_tokens: int, block_size: int = 64,
                  dtype=torch.float32, device="cpu"):
         """``row_dims[i]`` is the row width of stream ``i``;
-        ``state_shapes[name]`` the per-slot shape of a carried state.
+        ``state_shapes[name]`` the per-slot shape of a carried state, or
+        ``(shape, dtype)`` for a state kept in another number format than
+        the pools (a recurrence's fp32 matrix beside 16-bit rows).
         ``max_tokens`` bounds the tokens live at once (each sequence rounded
         up to whole blocks)."""
         self.block_size = block_size
@@ -72,9 +74,13 @@ class PagedStateCache:
         self.dtype = dtype
         self.pools = [torch.zeros(self.num_blocks, block_size, d, dtype=dtype,
                                   device=device) for d in row_dims]
-        self.states = {k: torch.zeros((num_slots,) + tuple(s), dtype=dtype,
-                                      device=device)
-                       for k, s in state_shapes.items()}
+        self.states = {}
+        for k, s in state_shapes.items():
+            sdt = dtype
+            if len(s) == 2 and isinstance(s[1], torch.dtype):
+                s, sdt = s
+            self.states[k] = torch.zeros((num_slots,) + tuple(s), dtype=sdt,
+                                         device=device)
         self.free_blocks = list(range(self.num_blocks - 1, -1, -1))
         self.block_table: Dict[int, List[int]] = {s: [] for s in
                                                   range(num_slots)}

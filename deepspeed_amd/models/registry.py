@@ -3,7 +3,9 @@ model class, the way ``init_inference`` users expect from Hugging Face style
 folders.
 
 ``register_architecture(name, build)`` adds a builder
-``build(config_dict, dtype) -> nn.Module``; the module may define
+``build(config_dict, dtype) -> nn.Module`` (with ``wants_tensors=True`` it is
+called as ``build(config_dict, dtype, tensors)`` so sizes that only tensor
+shapes give can be read; ``tensors`` is None without a checkpoint); the module may define
 ``load_named_tensors(dict)`` to take checkpoint tensors under their file
 names (otherwise ``load_state_dict`` is used). ``load_pretrained(folder)``
 reads config.json + *.safetensors and returns the model on ``device``.
@@ -18,10 +20,16 @@ from typing import Callable, Dict
 import torch
 
 _BUILDERS: Dict[str, Callable] = {}
+_WANTS_TENSORS = set()
 
 
-def register_architecture(name: str, build: Callable):
+def register_architecture(name: str, build: Callable,
+                          wants_tensors: bool = False):
     _BUILDERS[name] = build
+    if wants_tensors:
+        _WANTS_TENSORS.add(name)
+    else:
+        _WANTS_TENSORS.discard(name)
 
 
 def architectures():
@@ -37,11 +45,13 @@ def _arch_name(cfg: dict) -> str:
     return name
 
 
-def build_model(cfg: dict, dtype=torch.bfloat16):
+def build_model(cfg: dict, dtype=torch.bfloat16, tensors=None):
     name = _arch_name(cfg)
     if name not in _BUILDERS:
         raise ValueError(f"unknown architecture {name!r}; known: "
                          f"{architectures()}")
+    if name in _WANTS_TENSORS:
+        return _BUILDERS[name](cfg, dtype, tensors)
     return _BUILDERS[name](cfg, dtype)
 
 
@@ -49,12 +59,12 @@ def load_pretrained(folder: str, dtype=torch.bfloat16, device="cpu"):
     from safetensors.torch import load_file
     with open(os.path.join(folder, "config.json")) as f:
         cfg = json.load(f)
-    model = build_model(cfg, dtype)
     tensors = {}
     for path in sorted(glob.glob(os.path.join(folder, "*.safetensors"))):
         tensors.update(load_file(path))
     if not tensors:
         raise FileNotFoundError(f"no *.safetensors under {folder}")
+    model = build_model(cfg, dtype, tensors)
     if hasattr(model, "load_named_tensors"):
         model.load_named_tensors(tensors)
     else:
@@ -80,6 +90,7 @@ def _dataclass_builder(config_cls, model_cls, rename=None):
 def _register_builtin():
     from .fizesun import FizesunConfig, FizesunForCausalLM
     from .llama import LlamaConfig, LlamaForCausalLM
+    from .lolulorn import build_from_config as build_lolulorn
     from .mixtral import MixtralConfig, MixtralForCausalLM
     hf = {"num_hidden_layers": "num_layers",
           "num_attention_heads": "num_heads",
@@ -96,6 +107,7 @@ def _register_builtin():
     register_architecture(
         "Fizesun", lambda cfg, dtype: FizesunForCausalLM(
             FizesunConfig.from_dict(cfg), dtype))
+    register_architecture("Lolulorn", build_lolulorn, wants_tensors=True)
 
 
 _register_builtin()

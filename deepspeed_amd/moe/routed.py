@@ -1,8 +1,11 @@
 """Serving-side mixture of experts: no capacity, no token dropping.
 
 ``topk_softmax`` picks each token's ``top`` largest router logits and weights
-them by a softmax over the CHOSEN logits only (fp32). ``RoutedExperts`` runs
-clamped-SwiGLU experts: tokens are grouped by expert, each expert is one pair
+them by a softmax over the CHOSEN logits only (fp32).
+``grouped_sigmoid_topk`` scores experts by ``sigmoid(logit)``, chooses among
+the experts of the best few groups by score plus a per-expert correction, and
+weights the chosen ones by their uncorrected scores. ``RoutedExperts`` runs
+gated experts (clamped SwiGLU or plain SiLU gating): tokens are grouped by expert, each expert is one pair
 of vendor GEMMs on its contiguous group, and a combine kernel sums a token's
 weighted expert outputs (plus an optional shared expert scaled by a per-token
 sigmoid gate) in fp32. Training-time MoE with capacity and all-to-all lives
@@ -13,7 +16,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from ..ops.activations import clamped_swiglu
+from ..ops.activations import clamped_swiglu, glu
 
 
 def _sk():
@@ -27,6 +30,33 @@ def topk_softmax(logits, top):
         return _sk().topk_softmax(logits.float(), top)
     val, idx = torch.topk(logits.float(), top, dim=-1)
     return idx, torch.softmax(val, dim=-1)
+
+
+def grouped_sigmoid_topk(logits, correction, top, groups=1, keep=1):
+    """logits [T, E] fp32, correction [E] fp32. Scores ``s = sigmoid(logits)``;
+    choice scores ``c = s + correction``. The E experts form ``groups`` equal
+    runs of neighbours; a group's score is the sum of its two largest choice
+    scores (its only one when groups hold one expert) and only experts of the
+    ``keep`` best groups can be chosen. Returns the ``top`` allowed experts
+    with the largest choice scores (idx [T, top] int64) and their weights
+    ``s[idx]`` (fp32, not renormalised)."""
+    T, E = logits.shape
+    assert E % groups == 0 and 1 <= keep <= groups
+    assert top <= keep * (E // groups), "more picks than allowed experts"
+    if logits.is_cuda and _sk().enabled():
+        return _sk().grouped_sigmoid_topk(logits.float(), correction, top,
+                                          groups, keep)
+    s = torch.sigmoid(logits.float())
+    c = s + correction.float()
+    if groups > 1:
+        per = c.view(T, groups, E // groups)
+        gs = per.topk(min(2, E // groups), dim=-1).values.sum(-1)
+        best = gs.topk(keep, dim=-1).indices
+        allowed = torch.zeros(T, groups, dtype=torch.bool, device=c.device)
+        allowed.scatter_(1, best, True)
+        c = per.masked_fill(~allowed[:, :, None], float("-inf")).view(T, E)
+    idx = c.topk(top, dim=-1).indices
+    return idx, s.gather(1, idx)
 
 
 def moe_combine(y, inv, weight, shared=None, shared_gate=None):
@@ -60,10 +90,22 @@ class ClampedGLUExpert(nn.Module):
 
 
 class RoutedExperts(nn.Module):
-    def __init__(self, width, ff, experts, top, limit, shared_ff=0,
-                 shared_limit=0.0, dtype=torch.float32):
+    """``activation``: "clamped_swiglu" (with ``limit``) or a gate name of
+    ``ops.activations.glu`` ("silu", "gelu_tanh"). ``router``: "softmax"
+    (``topk_softmax`` of logits + ``router_bias``) or "sigmoid_grouped"
+    (``grouped_sigmoid_topk`` with ``groups = (count, keep)`` and
+    ``router_bias`` as the choice correction)."""
+
+    def __init__(self, width, ff, experts, top, limit=0.0, shared_ff=0,
+                 shared_limit=0.0, dtype=torch.float32,
+                 activation="clamped_swiglu", router="softmax",
+                 groups=(1, 1)):
         super().__init__()
         self.experts, self.top, self.limit = experts, top, float(limit)
+        self.activation, self.router_kind = activation, router
+        self.groups = (int(groups[0]), int(groups[1]))
+        if router not in ("softmax", "sigmoid_grouped"):
+            raise ValueError(f"unknown router {router!r}")
         self.router = nn.Parameter(torch.empty(experts, width,
                                                dtype=torch.float32),
                                    requires_grad=False)
@@ -82,19 +124,30 @@ class RoutedExperts(nn.Module):
             self.shared_gate = nn.Parameter(torch.empty(1, width, dtype=dtype),
                                             requires_grad=False)
 
+    def _act(self, gu):
+        if self.activation == "clamped_swiglu":
+            return clamped_swiglu(gu, self.limit)
+        return glu(gu, self.activation)
+
+    def route(self, h):
+        if self.router_kind == "softmax":
+            logits = F.linear(h.float(), self.router.float(),
+                              self.router_bias.float())
+            return topk_softmax(logits, self.top)
+        logits = F.linear(h.float(), self.router.float())
+        return grouped_sigmoid_topk(logits, self.router_bias, self.top,
+                                    *self.groups)
+
     def forward(self, h):
         T = h.shape[0]
-        logits = F.linear(h.float(), self.router.float(),
-                          self.router_bias.float())
-        idx, weight = topk_softmax(logits, self.top)
+        idx, weight = self.route(h)
         picks = T * self.top
         if picks <= self.DENSE_MAX_PICKS and 2 * picks >= self.experts:
             # decode-sized steps: run every expert on every token as three
             # batched GEMMs (the picks of a few tokens touch most experts'
             # weights anyway) and pick the chosen outputs; no host round trip
-            mid = clamped_swiglu(torch.bmm(h.expand(self.experts, T, -1),
-                                           self.w_gu.transpose(1, 2)),
-                                 self.limit)
+            mid = self._act(torch.bmm(h.expand(self.experts, T, -1),
+                                      self.w_gu.transpose(1, 2)))
             y = torch.bmm(mid, self.w_down.transpose(1, 2)) \
                 .reshape(self.experts * T, -1)
             inv = idx * T + torch.arange(T, device=h.device)[:, None]
@@ -123,8 +176,7 @@ class RoutedExperts(nn.Module):
         at = 0
         for e, n in enumerate(counts):
             if n:
-                mid = clamped_swiglu(F.linear(xs[at:at + n], self.w_gu[e]),
-                                     self.limit)
+                mid = self._act(F.linear(xs[at:at + n], self.w_gu[e]))
                 y[at:at + n] = F.linear(mid, self.w_down[e])
                 at += n
         return y, inv.view(T, self.top)

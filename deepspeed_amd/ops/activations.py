@@ -6,7 +6,9 @@
 * ``clamped_swiglu(gu, limit)``: with ``g = min(gate, limit)`` and
   ``u = clamp(up, -limit, limit)``: ``g * sigmoid(1.702 g) * (u + 1)``;
   ``gu`` holds gate and up side by side ([T, 2F] -> [T, F]).
-Both evaluate in fp32 and round once.
+* ``glu(gu, act)``: ``act(gate) * up`` with ``act`` "silu" or "gelu_tanh"
+  (``0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))``), same layout.
+All evaluate in fp32 and round once.
 """
 
 import torch
@@ -41,3 +43,18 @@ def clamped_swiglu(gu, limit):
     g = gu[..., :f].float().clamp(max=limit)
     u = gu[..., f:].float().clamp(-limit, limit)
     return (g * torch.sigmoid(SWISH_SLOPE * g) * (u + 1)).to(gu.dtype)
+
+
+GLU_ACTS = ("silu", "gelu_tanh")
+
+
+def glu(gu, act):
+    """gu [..., 2F] = gate | up -> act(gate) * up as [..., F]."""
+    if act not in GLU_ACTS:
+        raise ValueError(f"unknown gate activation {act!r}")
+    if gu.is_cuda and _sk().enabled():
+        return _sk().glu(gu, GLU_ACTS.index(act))
+    f = gu.shape[-1] // 2
+    g, u = gu[..., :f].float(), gu[..., f:].float()
+    a = F.silu(g) if act == "silu" else F.gelu(g, approximate="tanh")
+    return (a * u).to(gu.dtype)

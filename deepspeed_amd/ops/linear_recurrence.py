@@ -1,0 +1,125 @@
+"""Linear recurrences with a matrix state per head, for ragged batches.
+
+A head carries ``S`` ([dim, vdim], fp32, one per request slot). Per token, in
+this order:
+
+    S <- decay * S                  decay: one number per head, or one per key
+                                    channel (it then scales the rows of S)
+    u  = v                          plain form ("gla")
+    u  = beta * (v - S^T k)         delta-rule form (beta given)
+    S <- S + k u^T
+    o  = S^T q                      (sees this token's write)
+
+so a step that brings only a portion of a sequence continues from the slot's
+state exactly where the previous step stopped, and a result cannot depend on
+where a sequence was cut. Everything is fp32; q/k/v may arrive in the compute
+dtype (they are projections) and are widened on load.
+
+Around the scan:
+
+* ``delta_prep``: the gated delta rule's inputs from its fused projection
+  (short convolution + SiLU on q, k, v with carried tails; q and k scaled to
+  unit length per head; ``beta = sigmoid(b)``;
+  ``decay = exp(-exp(A_log) * softplus(a + dt_bias))``).
+* ``sigmoid_pow``: ``sigmoid(z + bias) ** (1 / tau)`` for per-channel decays.
+* ``head_norm_gate``: per-head RMS norm of the read-out times a weight shared
+  by the heads, times ``silu(gate)``.
+"""
+
+import torch
+import torch.nn.functional as F
+
+from .causal_conv import conv_silu_ragged
+
+UNIT_EPS = 1e-6
+
+
+def _sk():
+    from . import serving_kernels
+    return serving_kernels
+
+
+def unit_heads(x, scale=1.0):
+    """x [T, n, d] fp32 -> x / sqrt(sum(x^2) + 1e-6) * scale per head."""
+    return x * torch.rsqrt(x.pow(2).sum(-1, keepdim=True) + UNIT_EPS) * scale
+
+
+def delta_prep(proj, batch, conv_w, conv_state, a_log, dt_bias, kv_heads,
+               heads, dim, vdim):
+    """proj [T, 2*kv_heads*dim + 2*heads*vdim + 2*heads] =
+    q | k | v | gate | b | a (the gate columns are left for
+    ``head_norm_gate``). conv_w [2*kv_heads*dim + heads*vdim, taps] and
+    conv_state [slots, taps-1, same] cover the q|k|v columns.
+    Returns fp32 q [T, kv_heads, dim] (unit length times dim^-1/2),
+    k [T, kv_heads, dim] (unit length), v [T, heads, vdim], beta [T, heads],
+    decay [T, heads]."""
+    T = proj.shape[0]
+    nqk, nv = kv_heads * dim, heads * vdim
+    C = 2 * nqk + nv
+    assert proj.shape[1] == C + nv + 2 * heads and conv_w.shape[0] == C
+    if proj.is_cuda and _sk().enabled():
+        return _sk().delta_prep(proj, batch, conv_w, conv_state, a_log,
+                                dt_bias, kv_heads, heads, dim, vdim)
+    y = conv_silu_ragged(proj[:, :C], conv_w, conv_state, batch)
+    q = unit_heads(y[:, :nqk].reshape(T, kv_heads, dim), dim ** -0.5)
+    k = unit_heads(y[:, nqk:2 * nqk].reshape(T, kv_heads, dim))
+    v = y[:, 2 * nqk:].reshape(T, heads, vdim)
+    beta = torch.sigmoid(proj[:, C + nv:C + nv + heads].float())
+    dt = F.softplus(proj[:, C + nv + heads:].float() + dt_bias.float())
+    decay = torch.exp(-torch.exp(a_log.float()) * dt)
+    return q.contiguous(), k.contiguous(), v.contiguous(), beta, decay
+
+
+def sigmoid_pow(z, bias, inv_tau):
+    """``sigmoid(z + bias) ** inv_tau`` in fp32, evaluated as
+    ``exp(inv_tau * log_sigmoid(.))``."""
+    if z.is_cuda and _sk().enabled():
+        return _sk().sigmoid_pow(z, bias, inv_tau)
+    return torch.exp(inv_tau * F.logsigmoid(z.float() + bias.float()))
+
+
+def linear_scan(q, k, v, decay, beta, state, batch, q_scale=1.0):
+    """q, k [T, G, dim]; v [T, H, vdim] (head h reads q/k head h // (H/G));
+    decay [T, H] or [T, H, dim] fp32; beta [T, H] fp32 or None;
+    state [slots, H, dim, vdim] fp32, updated in place. q, k, v may be
+    strided views (last axis contiguous). Returns o [T, H, vdim] fp32."""
+    T, G, dim = q.shape
+    H, vdim = v.shape[1], v.shape[2]
+    assert H % G == 0 and state.dtype == torch.float32
+    assert state.shape[1:] == (H, dim, vdim)
+    assert decay.shape in ((T, H), (T, H, dim))
+    if q.is_cuda and _sk().enabled():
+        return _sk().linear_scan(q, k, v, decay, beta, state, batch, q_scale)
+    rep = H // G
+    qf = (q.float() * q_scale).repeat_interleave(rep, 1)
+    kf = k.float().repeat_interleave(rep, 1)
+    vf = v.float()
+    dec = decay.float()
+    dec = dec[:, :, None, None] if dec.dim() == 2 else dec[:, :, :, None]
+    out = torch.empty(T, H, vdim, dtype=torch.float32, device=q.device)
+    at = 0
+    for slot, count in zip(batch.slots, batch.counts):
+        S = state[slot]
+        for t in range(at, at + count):
+            S = dec[t] * S
+            u = vf[t]
+            if beta is not None:
+                u = beta[t, :, None] * (u - torch.einsum("hdv,hd->hv", S,
+                                                         kf[t]))
+            S = S + kf[t][:, :, None] * u[:, None, :]
+            out[t] = torch.einsum("hdv,hd->hv", S, qf[t])
+        state[slot] = S
+        at += count
+    return out
+
+
+def head_norm_gate(o, weight, gate, eps, out_dtype):
+    """o [T, H, vdim] fp32; weight [vdim]; gate [T, H*vdim] pre-activation
+    (may be a column slice). Returns
+    ``o / sqrt(mean_v(o^2) + eps) * weight * silu(gate)`` as
+    [T, H*vdim] ``out_dtype``."""
+    T, H, vdim = o.shape
+    if o.is_cuda and _sk().enabled():
+        return _sk().head_norm_gate(o, weight, gate, eps, out_dtype)
+    y = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * weight.float()
+    return (y.reshape(T, H * vdim) * F.silu(gate.float())).to(out_dtype)

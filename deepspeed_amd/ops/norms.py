@@ -170,3 +170,43 @@ class ScalarRMSNorm(torch.nn.Module):
 
     def forward(self, x, out_dtype=None, index=None):
         return scalar_rms_norm(x, self.gain, self.eps, out_dtype, index)
+
+
+def layer_norm_add_(x, y, weight, bias, eps, out_dtype=None):
+    """Post-sublayer norm on an fp32 residual stream, in place:
+    ``x += (y - mean) / sqrt(var + eps) * weight + bias`` with the statistics
+    of each row of ``y`` ([T, C], any float type) in fp32 and ``var`` the mean
+    squared deviation. With ``out_dtype`` the same pass also returns the new
+    ``x`` rounded to that type (the next sublayer's GEMM operand); otherwise
+    it returns ``x``."""
+    assert x.dtype == torch.float32 and x.shape == y.shape
+    if x.is_cuda and _sk().enabled():
+        return _sk().layer_norm_add(x, y, weight, bias, eps, out_dtype)
+    yf = y.float()
+    mu = yf.mean(-1, keepdim=True)
+    d = yf - mu
+    var = (d * d).mean(-1, keepdim=True)
+    x.add_(d * torch.rsqrt(var + eps) * weight.float() + bias.float())
+    return x if out_dtype in (None, torch.float32) else x.to(out_dtype)
+
+
+def layer_norm_rows(x, weight, bias, eps, out_dtype=None, index=None):
+    """Layer norm with weight and bias of the rows ``x[index]`` (all rows
+    without ``index``), fp32 statistics, rounded once to ``out_dtype``."""
+    out_dtype = out_dtype or x.dtype
+    if x.is_cuda and _sk().enabled():
+        return _sk().layer_norm_rows(x.contiguous(), weight, bias, eps,
+                                     out_dtype, index)
+    xf = (x if index is None else x[index]).float()
+    mu = xf.mean(-1, keepdim=True)
+    d = xf - mu
+    var = (d * d).mean(-1, keepdim=True)
+    return (d * torch.rsqrt(var + eps) * weight.float()
+            + bias.float()).to(out_dtype)
+
+
+def embed_rows(table, ids, scale, out_dtype=torch.float32):
+    """``table[ids] * scale`` in fp32, rounded once to ``out_dtype``."""
+    if table.is_cuda and _sk().enabled():
+        return _sk().embed_rows(table, ids, scale, out_dtype)
+    return (table[ids].float() * scale).to(out_dtype)

@@ -1,7 +1,7 @@
 """ctypes front-end of the ragged-batch serving kernels
-(csrc/serving/serving_kernels.hip -> deepspeed_amd/ops/_serving.so).
+(csrc/serving/*.hip -> deepspeed_amd/ops/_serving*.so).
 
-The library has a plain C ABI, so it builds with one hipcc call in a few
+The libraries have a plain C ABI, so each builds with one hipcc call in a few
 seconds and needs none of the torch headers; ``load()`` builds it on first use
 when it is missing or older than its source. Wrappers take torch tensors,
 check shapes and dtypes on the host (a kernel never sees operands it was not
@@ -20,56 +20,82 @@ import sys
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-SOURCE = os.path.join(_HERE, "csrc", "serving", "serving_kernels.hip")
-LIBRARY = os.path.join(_HERE, "_serving.so")
+_SRC = os.path.join(_HERE, "csrc", "serving")
+COMMON = os.path.join(_SRC, "serving_common.h")
+# One library per family of mechanisms, each built from one source file: a
+# model compiles and loads only the families its layers use.
+#   rows   : norms, short convolutions, residual adds, activations, routers
+#   latent : compressed-KV attention
+#   seq    : windowed multi-head attention over paged K/V, linear recurrences
+LIBRARIES = {
+    "rows": (os.path.join(_SRC, "serving_kernels.hip"),
+             os.path.join(_HERE, "_serving.so")),
+    "latent": (os.path.join(_SRC, "latent_kernels.hip"),
+               os.path.join(_HERE, "_serving_latent.so")),
+    "seq": (os.path.join(_SRC, "sequence_kernels.hip"),
+            os.path.join(_HERE, "_serving_seq.so")),
+}
+SOURCE, LIBRARY = LIBRARIES["rows"]
 HIPCC_FLAGS = ["-O3", "-std=c++17", "--offload-arch=gfx950",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
                "-shared", "-fPIC"]
 
-_lib = None
+_libs = {}
 
 
-def _compile(target):
+def _compile(source, target):
     hipcc = os.environ.get("HIPCC") or (
         "/opt/rocm/bin/hipcc" if os.path.exists("/opt/rocm/bin/hipcc")
         else "hipcc")
     tmp = "%s.%d.tmp" % (target, os.getpid())
-    cmd = [hipcc] + HIPCC_FLAGS + ["-o", tmp, SOURCE]
+    cmd = [hipcc] + HIPCC_FLAGS + ["-o", tmp, source]
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
                        text=True)
     if r.returncode != 0:
-        raise RuntimeError("building the serving kernels failed:\n" + r.stdout)
+        raise RuntimeError("building %s failed:\n%s"
+                           % (os.path.basename(source), r.stdout))
     os.replace(tmp, target)
     return target
 
 
-def _fresh(path):
+def _fresh(path, source):
     return os.path.exists(path) and \
-        os.path.getmtime(path) >= os.path.getmtime(SOURCE)
+        os.path.getmtime(path) >= max(os.path.getmtime(source),
+                                      os.path.getmtime(COMMON))
 
 
-def build(force=True):
-    """Compile the library in-tree (cross-compiles without a GPU). Returns the
-    path of the library to load. Where the tree cannot be written, a copy
-    keyed by the source's content goes to the temporary directory instead."""
-    if not force and _fresh(LIBRARY):
-        return LIBRARY
-    if os.access(os.path.dirname(LIBRARY), os.W_OK):
-        return _compile(LIBRARY)
-    import hashlib
-    import tempfile
-    with open(SOURCE, "rb") as f:
-        tag = hashlib.sha1(f.read()).hexdigest()[:16]
-    alt = os.path.join(tempfile.gettempdir(), "ds_amd_serving_%s.so" % tag)
-    return alt if os.path.exists(alt) else _compile(alt)
+def build(force=True, which=None):
+    """Compile the libraries in-tree (cross-compiles without a GPU); ``which``
+    names one family, default all. Returns the path of the (last) library.
+    Where the tree cannot be written, a copy keyed by the sources' content
+    goes to the temporary directory instead."""
+    path = None
+    for name in ([which] if which else list(LIBRARIES)):
+        source, library = LIBRARIES[name]
+        if not force and _fresh(library, source):
+            path = library
+        elif os.access(os.path.dirname(library), os.W_OK):
+            path = _compile(source, library)
+        else:
+            import hashlib
+            import tempfile
+            tag = hashlib.sha1()
+            for f in (COMMON, source):
+                with open(f, "rb") as fh:
+                    tag.update(fh.read())
+            alt = os.path.join(tempfile.gettempdir(), "ds_amd_serving_%s_%s.so"
+                               % (name, tag.hexdigest()[:16]))
+            path = alt if os.path.exists(alt) else _compile(source, alt)
+    return path
 
 
-def load():
-    global _lib
-    if _lib is None:
-        _lib = ctypes.CDLL(build(force=False))
-        _lib.dsv_latent_attn_lds.restype = ctypes.c_int64
-    return _lib
+def load(which="rows"):
+    lib = _libs.get(which)
+    if lib is None:
+        lib = _libs[which] = ctypes.CDLL(build(force=False, which=which))
+        if which == "latent":
+            lib.dsv_latent_attn_lds.restype = ctypes.c_int64
+    return lib
 
 
 def enabled() -> bool:
@@ -184,7 +210,7 @@ def latent_prep(proj, batch, pool, norm_w, eps, heads, dim, rot, rank,
     q_nope = torch.empty(heads, T, dim, dtype=dt, device=dev)
     q_rot = torch.empty(T, heads, rot, dtype=dt, device=dev)
     gate = torch.empty(T, heads, dtype=torch.float32, device=dev)
-    _check(load().dsv_latent_prep(
+    _check(load("latent").dsv_latent_prep(
         _p(proj), _i(proj.shape[1]), _p(_f32(norm_w)), _p(batch.tok_pos),
         _p(batch.tok_row), _p(cos), _p(sin), _p(pool), _p(q_nope), _p(q_rot),
         _p(gate), _i(_dt(proj)), _i(T), _i(heads), _i(dim), _i(rot), _i(rank),
@@ -195,7 +221,7 @@ def latent_prep(proj, batch, pool, norm_w, eps, heads, dim, rot, rank,
 def _attn_plan(batch, dtype, rank, rot):
     """Key-chunk length that fits LDS, and the number of key splits: few
     tokens over a long history are split so the launch still fills the chip."""
-    lib = load()
+    lib = load("latent")
     dt = _DT[dtype]
     kc = 64
     while kc > 4 and lib.dsv_latent_attn_lds(dt, rank, rot, kc) > 60 * 1024:
@@ -232,7 +258,7 @@ def latent_attention(q_lat, q_rot, pool, batch, rank, scale, path=None):
     assert q_lat.dtype == pool.dtype == q_rot.dtype
     assert q_rot.is_contiguous() and pool.is_contiguous()
     q_lat = q_lat.contiguous()
-    lib = load()
+    lib = load("latent")
     out = torch.empty_like(q_lat)
     mfma = q_lat.dtype == torch.bfloat16 and \
         lib.dsv_latent_attn_mfma_ok(_i(rank), _i(rot)) == 1
@@ -276,7 +302,7 @@ def gate_merge_heads(o, gate):
     H, T, v = o.shape
     assert gate.shape == (T, H) and gate.dtype == torch.float32
     out = torch.empty(T, H * v, dtype=o.dtype, device=o.device)
-    _check(load().dsv_gate_merge(_p(o.contiguous()), _p(gate), _p(out),
+    _check(load("latent").dsv_gate_merge(_p(o.contiguous()), _p(gate), _p(out),
                                  _i(_dt(o)), _i(T), _i(H), _i(v), _stream()),
            "gate_merge_heads")
     return out
@@ -328,6 +354,222 @@ def topk_softmax(logits, top):
                                    _i(T), _i(E), _i(top), _stream()),
            "topk_softmax")
     return idx, w
+
+
+# ------------------------------------------------- layer norm, embedding
+def layer_norm_add(x, y, weight, bias, eps, out_dtype=None):
+    """x += layer_norm(y) in place; returns the new x rounded to
+    ``out_dtype`` (x itself for fp32 / None)."""
+    T, C = x.shape
+    assert x.dtype == torch.float32 and x.is_contiguous()
+    assert y.shape == x.shape and weight.numel() == C and bias.numel() == C
+    y = y.contiguous()
+    copy = None
+    if out_dtype not in (None, torch.float32):
+        copy = torch.empty(T, C, dtype=out_dtype, device=x.device)
+    _check(load().dsv_layer_norm(
+        _p(y), _i(_dt(y)), _p(None), _p(_f32(weight)), _p(_f32(bias)), _p(x),
+        _p(copy), _i(0 if copy is None else _DT[out_dtype]), _i(1), _i(T),
+        _i(C), _f(eps), _stream()), "layer_norm_add")
+    return x if copy is None else copy
+
+
+def layer_norm_rows(x, weight, bias, eps, out_dtype, index=None):
+    rows = x.shape[0] if index is None else index.numel()
+    C = x.shape[1]
+    assert weight.numel() == C and bias.numel() == C
+    out = torch.empty(rows, C, dtype=out_dtype, device=x.device)
+    if index is not None:
+        index = index.to(torch.int64).contiguous()
+    _check(load().dsv_layer_norm(
+        _p(x), _i(_dt(x)), _p(index), _p(_f32(weight)), _p(_f32(bias)),
+        _p(None), _p(out), _i(_DT[out_dtype]), _i(0), _i(rows), _i(C),
+        _f(eps), _stream()), "layer_norm_rows")
+    return out
+
+
+def embed_rows(table, ids, scale, out_dtype=torch.float32):
+    assert table.is_contiguous() and table.dim() == 2
+    ids = ids.to(torch.int64).contiguous()
+    out = torch.empty(ids.numel(), table.shape[1], dtype=torch.float32,
+                      device=table.device)
+    _check(load().dsv_embed_rows(_p(table), _i(_dt(table)), _p(ids), _p(out),
+                                 _i(ids.numel()), _i(table.shape[1]),
+                                 _f(scale), _stream()), "embed_rows")
+    return out if out_dtype == torch.float32 else out.to(out_dtype)
+
+
+def glu(gu, act):
+    gu = gu.contiguous()
+    F = gu.shape[-1] // 2
+    rows = gu.numel() // (2 * F)
+    out = torch.empty(gu.shape[:-1] + (F,), dtype=gu.dtype, device=gu.device)
+    _check(load().dsv_glu(_p(gu), _p(out), _i(_dt(gu)), _l(rows), _i(F),
+                          _i(act), _stream()), "glu")
+    return out
+
+
+def grouped_sigmoid_topk(logits, correction, top, groups, keep):
+    T, E = logits.shape
+    assert logits.dtype == torch.float32 and correction.numel() == E
+    idx = torch.empty(T, top, dtype=torch.int64, device=logits.device)
+    w = torch.empty(T, top, dtype=torch.float32, device=logits.device)
+    _check(load().dsv_grouped_sigmoid_topk(
+        _p(logits.contiguous()), _p(_f32(correction).contiguous()), _p(idx),
+        _p(w), _i(T), _i(E), _i(top), _i(groups), _i(keep), _stream()),
+        "grouped_sigmoid_topk")
+    return idx, w
+
+
+# ------------------------------------------------------ windowed attention
+def _seq():
+    lib = load("seq")
+    lib.dsv_window_attn_lds.restype = ctypes.c_int64
+    return lib
+
+
+def _rows_ok(t):
+    """A 2-d operand whose rows are contiguous (a column slice is fine)."""
+    assert t.is_cuda and t.dim() == 2 and t.stride(1) == 1
+    return t
+
+
+def attn_prep(proj, batch, pool, q_norm_w, k_norm_w, eps, heads, kv_heads,
+              dim, vdim, rot_dims, cos, sin, own_kv=True):
+    T = proj.shape[0]
+    assert proj.is_contiguous() and proj.dtype == pool.dtype
+    assert T == batch.n_tokens and q_norm_w.numel() == heads * dim
+    assert pool.shape[-1] == kv_heads * (dim + vdim) and pool.is_contiguous()
+    assert rot_dims % 2 == 0 and rot_dims <= dim
+    assert cos.shape[1] == rot_dims // 2 and cos.shape[0] >= batch.max_ctx
+    assert cos.dtype == torch.float32 and sin.shape == cos.shape
+    if own_kv:
+        assert k_norm_w.numel() == kv_heads * dim
+    q = torch.empty(T, heads, dim, dtype=proj.dtype, device=proj.device)
+    _check(_seq().dsv_attn_prep(
+        _p(proj), _i(proj.shape[1]), _p(_f32(q_norm_w)),
+        _p(_f32(k_norm_w) if own_kv else None), _p(batch.tok_pos),
+        _p(batch.tok_row), _p(cos), _p(sin), _p(pool), _p(q), _i(_dt(proj)),
+        _i(T), _i(heads), _i(kv_heads), _i(dim), _i(vdim), _i(rot_dims),
+        _i(1 if own_kv else 0), _f(eps), _stream()), "attn_prep")
+    return q
+
+
+def window_attention(q, pool, batch, kv_heads, dim, vdim, scale, window=0,
+                     keep_first=0, path=None):
+    T, H, d = q.shape
+    assert d == dim and T == batch.n_tokens and q.is_contiguous()
+    assert pool.shape[1] == batch.block_size and pool.is_contiguous()
+    assert q.dtype == pool.dtype
+    lib = _seq()
+    dt = _dt(q)
+    kc = 64
+    while kc > 4 and lib.dsv_window_attn_lds(dt, dim, vdim, kc) > 60 * 1024:
+        kc //= 2
+    # few tokens over a long visible range (decoding): split the keys so the
+    # launch still covers the chip; partial sums are merged in fp32
+    reach = batch.max_ctx if window <= 0 else \
+        min(batch.max_ctx, window + keep_first)
+    nsplit = 1
+    if T * kv_heads <= 128:
+        nsplit = max(1, min(32, reach // (4 * kc),
+                            1024 // max(1, T * kv_heads)))
+    out = torch.empty(T, H, vdim, dtype=q.dtype, device=q.device)
+    part = None
+    if nsplit > 1:
+        part = torch.empty(T, nsplit, H, vdim + 2, dtype=torch.float32,
+                           device=q.device)
+    _check(lib.dsv_window_attn(
+        _p(q), _p(pool), _p(batch.tok_seq), _p(batch.tok_pos),
+        _p(batch.block_table), _i(batch.block_table.shape[1]),
+        _i(batch.block_size), _p(out), _p(part), _i(dt), _i(T), _i(H),
+        _i(kv_heads), _i(dim), _i(vdim), _i(kc), _i(nsplit), _f(scale),
+        _i(window), _i(keep_first), _stream()), "window_attention")
+    return out.view(T, H * vdim)
+
+
+# ------------------------------------------------------ linear recurrences
+def delta_prep(proj, batch, conv_w, conv_state, a_log, dt_bias, kv_heads,
+               heads, dim, vdim):
+    T = proj.shape[0]
+    taps = conv_w.shape[1]
+    C = 2 * kv_heads * dim + heads * vdim
+    assert proj.is_contiguous() and T == batch.n_tokens
+    assert conv_w.dtype == proj.dtype == conv_state.dtype
+    assert conv_w.is_contiguous() and conv_w.shape[0] == C
+    assert conv_state.shape[1:] == (taps - 1, C)
+    assert conv_state.stride(2) == 1 and (taps == 1
+                                          or conv_state.stride(1) == C)
+    dev = proj.device
+    f32 = dict(dtype=torch.float32, device=dev)
+    q = torch.empty(T, kv_heads, dim, **f32)
+    k = torch.empty(T, kv_heads, dim, **f32)
+    v = torch.empty(T, heads, vdim, **f32)
+    beta = torch.empty(T, heads, **f32)
+    decay = torch.empty(T, heads, **f32)
+    _check(_seq().dsv_delta_prep(
+        _p(proj), _i(proj.shape[1]), _p(conv_w),
+        ctypes.c_void_p(conv_state.data_ptr()), _l(conv_state.stride(0)),
+        _p(batch.cu), _p(batch.seq_slot), _p(batch.seq_start),
+        _p(batch.tok_seq), _p(batch.tok_pos), _p(_f32(a_log)),
+        _p(_f32(dt_bias)), _p(q), _p(k), _p(v), _p(beta), _p(decay),
+        _i(_dt(proj)), _i(T), _i(batch.n_seqs), _i(kv_heads), _i(heads),
+        _i(dim), _i(vdim), _i(taps), _stream()), "delta_prep")
+    return q, k, v, beta, decay
+
+
+def sigmoid_pow(z, bias, inv_tau):
+    z = z.contiguous()
+    C = z.shape[-1]
+    assert bias.numel() == C
+    out = torch.empty(z.shape, dtype=torch.float32, device=z.device)
+    _check(_seq().dsv_sigmoid_pow(_p(z), _p(_f32(bias)), _p(out), _i(_dt(z)),
+                                  _l(z.numel()), _i(C), _f(inv_tau),
+                                  _stream()), "sigmoid_pow")
+    return out
+
+
+def _heads_view(t):
+    """[T, n, d] whose heads are side by side in a row: row stride."""
+    assert t.is_cuda and t.stride(2) == 1 and t.stride(1) == t.shape[2]
+    return ctypes.c_void_p(t.data_ptr()), _i(t.stride(0))
+
+
+def linear_scan(q, k, v, decay, beta, state, batch, q_scale=1.0):
+    T, G, dim = q.shape
+    H, vdim = v.shape[1], v.shape[2]
+    assert q.dtype == k.dtype == v.dtype and k.shape == q.shape
+    assert T == batch.n_tokens and v.shape[0] == T
+    assert state.dtype == torch.float32 and state.is_contiguous()
+    assert state.shape[1:] == (H, dim, vdim)
+    assert decay.dtype == torch.float32 and decay.is_contiguous()
+    channel = decay.dim() == 3
+    assert decay.shape == ((T, H, dim) if channel else (T, H))
+    if beta is not None:
+        assert beta.shape == (T, H) and beta.dtype == torch.float32
+        beta = beta.contiguous()
+    out = torch.empty(T, H, vdim, dtype=torch.float32, device=q.device)
+    (qp, ldq), (kp, ldk), (vp, ldv) = (_heads_view(t) for t in (q, k, v))
+    _check(_seq().dsv_linear_scan(
+        qp, ldq, kp, ldk, vp, ldv, _p(decay), _i(1 if channel else 0),
+        _p(beta), _p(state), _p(batch.cu), _p(batch.seq_slot), _p(out),
+        _i(_dt(q)), _i(batch.n_seqs), _i(G), _i(H), _i(dim), _i(vdim),
+        _f(q_scale), _stream()), "linear_scan")
+    return out
+
+
+def head_norm_gate(o, weight, gate, eps, out_dtype):
+    T, H, vdim = o.shape
+    assert o.dtype == torch.float32 and o.is_contiguous()
+    assert weight.numel() == vdim and gate.shape == (T, H * vdim)
+    assert gate.dtype == out_dtype
+    _rows_ok(gate)
+    out = torch.empty(T, H * vdim, dtype=out_dtype, device=o.device)
+    _check(_seq().dsv_head_norm_gate(
+        _p(o), _p(_f32(weight)), ctypes.c_void_p(gate.data_ptr()),
+        _i(gate.stride(0)), _p(out), _i(_DT[out_dtype]), _i(T), _i(H),
+        _i(vdim), _f(eps), _stream()), "head_norm_gate")
+    return out
 
 
 if __name__ == "__main__":
