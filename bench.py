@@ -34,7 +34,7 @@ def parse_args():
                    help="ZeRO-Offload optimizer states to host DRAM")
     p.add_argument("--activation-checkpointing", action="store_true")
     p.add_argument("--local_rank", type=int, default=-1)
-    p.add_argument("--serving", type=str, default=None, choices=["fizesun"],
+    p.add_argument("--serving", type=str, default=None, choices=["fizesun", "lolulorn"],
                    help="instead of the training step: serving throughput "
                         "(prefill, decode) of this design beside Llama at "
                         "equal size, with per-kernel roofline distances")
@@ -76,7 +76,7 @@ def main():
     args = parse_args()
     if args.serving:
         from deepspeed_amd.inference.serving_bench import main as serving
-        serving(args.serving_sizes, args.serving_out)
+        serving(args.serving_sizes, args.serving_out, args.serving)
         return
     world_size = int(os.environ.get("WORLD_SIZE", 1))
     rank = int(os.environ.get("RANK", 0))

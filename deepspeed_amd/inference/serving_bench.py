@@ -8,6 +8,10 @@ Random weights, synthetic tokens, bf16, one GPU. For every size:
   same shapes, timed alone, against max(bytes / HBM bandwidth, flops / MFMA
   peak). "distance" is measured time over that bound.
 Run through ``python bench.py --serving fizesun``.
+
+``--serving lolulorn`` does the same for Lolulorn (one block of gla /
+attention / attention on borrowed rows / delta layers, dense and routed
+feed-forwards) beside Llama, with Fizesun's throughput for the ragged path.
 """
 
 import json
@@ -249,6 +253,246 @@ def _kernel_rows(z, dev):
     return out
 
 
+# ------------------------------------------------------------- Lolulorn
+def lolulorn_config(z, vocab=32000):
+    """One block [gla, attention, attention on the rows of the one before,
+    delta] repeated to ``layers``; attention heads of 128 with 4 query heads
+    per key/value head and a window of 1024 that keeps 4 first tokens;
+    recurrent heads with keys of 128 and values of 256."""
+    H = z["heads"]
+    att = {"heads": H, "kv_heads": max(1, H // 4), "dim": 128, "vdim": 128,
+           "scale": 128 ** -0.5, "mask": {"size": 1024, "keep_first": 4},
+           "rot": {"base": 10000.0, "dims": 64, "scaling": {"factor": 2.0}}}
+    gla = {"heads": max(1, H // 2), "dim": 128, "vdim": 256, "tau": 16.0,
+           "rank": 16}
+    delta = {"heads": max(1, H // 2), "kv_heads": max(1, H // 4), "dim": 128,
+             "vdim": 256, "conv": 4}
+    dense = {"kind": "dense", "ff": z["ff"]}
+    moe = {"kind": "moe", "expert": {"ff": z["eff"]},
+           "router": {"experts": z["experts"], "top": z["top"],
+                      "groups": {"count": 4, "keep": 2}}}
+    layers = []
+    for i in range(z["layers"]):
+        kind = i % 4
+        if kind == 0:
+            layers.append({"type": "gla", "mixer": gla, "mlp": dense})
+        elif kind == 1:
+            layers.append({"type": "attention", "mixer": att, "mlp": moe})
+        elif kind == 2:
+            layers.append({"type": "attention",
+                           "mixer": {**att, "kv_from": i - 1}, "mlp": dense})
+        else:
+            layers.append({"type": "delta", "mixer": delta, "mlp": moe})
+    return {"architecture": "Lolulorn", "vocab": vocab, "width": z["width"],
+            "norm": {"eps": 1e-6}, "embedding": {"scale": 1.0},
+            "layers": layers}
+
+
+def _ragged_throughput(cfg, z, dev):
+    from ..models.registry import build_model
+    from .ragged import ContinuousBatcher
+    model = build_model(cfg, torch.bfloat16).init_random(0).to(dev).eval()
+    B, S = z["batch"], z["seq"]
+    b = ContinuousBatcher(model, max_slots=B, dtype=torch.bfloat16,
+                          device=dev, max_tokens=B * (S + 64))
+    g = torch.Generator().manual_seed(0)
+    prompts = torch.randint(0, 32000, (B, S), generator=g).tolist()
+
+    def prefill():
+        reqs = [b.open(i) for i in range(B)]
+        b.feed([(r, p) for r, p in zip(reqs, prompts)], rows=[0])
+        return reqs
+
+    def prefill_and_close():
+        for r in prefill():
+            b.close(r)
+
+    t_pre = _timed(prefill_and_close, 1, 3)
+    reqs = prefill()
+
+    def decode():
+        b.feed([(r, [7]) for r in reqs], rows=list(range(B)))
+
+    t_dec = _timed(decode, 3, 20)
+    for r in reqs:
+        b.close(r)
+    del model, b
+    torch.cuda.empty_cache()
+    return {"prefill_tok_s": B * S / t_pre, "decode_tok_s": B / t_dec,
+            "decode_ms": 1e3 * t_dec}
+
+
+@torch.no_grad()
+def _lolulorn_kernel_rows(z, dev):
+    """(name, like, seconds, bound seconds) per Lolulorn kernel at this size,
+    each followed by the like kernel of the Llama path."""
+    from ..ops import serving_kernels as sk
+    from ..ops.attention import flash_attn_available, flash_attn_fwd
+    from ..ops.norms import rms_norm
+    from ..ops.paged_attention import paged_decode_attention
+    from ..ops.rope import rope_tables
+    from ..ops.swiglu import swiglu
+    from .state_cache import PagedStateCache
+    bf = torch.bfloat16
+    B, S, W, H = z["batch"], z["seq"], z["width"], z["heads"]
+    F = z["ff"]
+    G, d, dv = max(1, H // 4), 128, 128
+    win, keep = 1024, 4
+    T = B * S
+    out = []
+
+    def row(name, like, fn, nbytes, flops=0.0, iters=5):
+        t = _timed(fn, 2, iters)
+        bound = max(nbytes / HBM_BW, flops / MFMA_BF16)
+        out.append({"kernel": name, "like": like, "us": 1e6 * t,
+                    "bound_us": 1e6 * bound, "distance": t / bound})
+
+    # ---- post-norm + residual against RMSNorm and the bf16 residual add
+    x32 = torch.randn(T, W, device=dev)
+    x16 = x32.to(bf)
+    y16 = (torch.randn(T, W, device=dev) * 0.01).to(bf)
+    wn = torch.ones(W, device=dev)
+    bn = torch.zeros(W, device=dev)
+    row("layer_norm_add (fp32 stream += LN(bf16), bf16 copy)", "rms_norm+add",
+        lambda: sk.layer_norm_add(x32, y16, wn, bn, 1e-6, bf), T * W * 12)
+    wn16 = wn.to(bf)
+    z16 = torch.empty_like(x16)
+    row("rms_norm + add (llama)", "",
+        lambda: torch.add(rms_norm(x16, wn16, 1e-6), y16, out=z16),
+        T * W * 10)
+    # ---- attention prologue and prefill
+    cache = PagedStateCache([G * (d + dv)], {}, B, B * (S + 64), dtype=bf,
+                            device=dev)
+    batch = cache.begin_ragged(list(range(B)), [S] * B)
+    cos, sin = rope_tables(64, cache.max_seq, 10000.0, device=dev, scaling=2.0)
+    proj = torch.randn(T, (H + 2 * G) * d, device=dev).to(bf)
+    qw, kw = torch.ones(H * d, device=dev), torch.ones(G * d, device=dev)
+    row("attn_prep (q/k norm, rotary, cache write)", "rms_norm",
+        lambda: sk.attn_prep(proj, batch, cache.pools[0], qw, kw, 1e-6, H, G,
+                             d, dv, 64, cos, sin, True),
+        T * (H + 2 * G) * d * 4)
+    p16 = torch.randn(T, (H + 2 * G) * d, device=dev).to(bf)
+    wp = torch.ones((H + 2 * G) * d, device=dev, dtype=bf)
+    row("rms_norm over the same columns (llama)", "",
+        lambda: rms_norm(p16, wp, 1e-6), T * (H + 2 * G) * d * 4)
+    q = sk.attn_prep(proj, batch, cache.pools[0], qw, kw, 1e-6, H, G, d, dv,
+                     64, cos, sin, True)
+    seen = sum(min(i + 1, win) + min(keep, max(0, i + 1 - win))
+               for i in range(S))
+    row("window_attention prefill (window %d + %d kept)" % (win, keep),
+        "flash_attn_fwd",
+        lambda: sk.window_attention(q, cache.pools[0], batch, G, d, dv,
+                                    d ** -0.5, win, keep),
+        T * H * (d + dv) * 2 + T * G * (d + dv) * 2,
+        2.0 * B * H * seen * (d + dv), iters=2)
+    qf = torch.randn(B, S, H, 128, device=dev).to(bf)
+    kf = torch.randn(B, S, G, 128, device=dev).to(bf)
+    if flash_attn_available(qf, kf):
+        row("flash_attn_fwd (llama, causal, no window)", "",
+            lambda: flash_attn_fwd(qf, kf, kf, causal=True),
+            (2 * qf.numel() + 2 * kf.numel()) * 2,
+            4.0 * B * H * (S * S / 2) * 128)
+    cache.end_step()
+    # ---- decode attention at B and at 64 requests
+    for NB in (B, 64):
+        big = PagedStateCache([G * (d + dv)], {}, NB, NB * (S + 64), dtype=bf,
+                              device=dev)
+        big.pools[0].normal_()
+        for i in range(NB):
+            big.lens[i] = S
+        bt = big.begin_ragged(list(range(NB)), [1] * NB)
+        qd = (torch.randn(NB, H, d, device=dev) * 0.1).to(bf)
+        vis = min(S + 1, win + keep)
+        row("window_attention decode, %d requests" % NB, "paged_decode",
+            lambda: sk.window_attention(qd, big.pools[0], bt, G, d, dv,
+                                        d ** -0.5, win, keep),
+            NB * vis * G * (d + dv) * 2)
+        big.end_step()
+        del big
+        nb = NB * ((S + 64) // 64)
+        kp = torch.randn(nb, G, 64, 128, device=dev).to(bf)
+        table = torch.arange(nb, dtype=torch.int32, device=dev).view(NB, -1)
+        lens = torch.full((NB,), S + 1, dtype=torch.int32, device=dev)
+        qp = torch.randn(NB, H, 128, device=dev).to(bf)
+        row("paged_decode, %d requests (llama, whole history)" % NB, "",
+            lambda: paged_decode_attention(qp, kp, kp, table, lens),
+            NB * (S + 1) * G * 128 * 2 * 2)
+        del kp
+    # ---- recurrences: no like kernel in the framework
+    RH, RG, rd, rv = max(1, H // 2), max(1, H // 4), 128, 256
+    for form in ("delta", "gla"):
+        g_ = RG if form == "delta" else RH
+        for NB, cnt in ((B, S), (B, 1), (64, 1)):
+            rc = PagedStateCache([], {"rec": ((RH, rd, rv), torch.float32)},
+                                 NB, NB * (S + 64), dtype=bf, device=dev)
+            bt = rc.begin_ragged(list(range(NB)), [cnt] * NB)
+            n = NB * cnt
+            if form == "delta":
+                qq = torch.randn(n, g_, rd, device=dev) * 0.1
+                kk = torch.nn.functional.normalize(
+                    torch.randn(n, g_, rd, device=dev), dim=-1)
+                vv = torch.randn(n, RH, rv, device=dev)
+                dec = torch.rand(n, RH, device=dev) * 0.1 + 0.9
+                beta = torch.rand(n, RH, device=dev)
+                io = n * (2 * g_ * rd + RH * rv) * 4
+            else:
+                qq = (torch.randn(n, g_, rd, device=dev) * 0.1).to(bf)
+                kk = (torch.randn(n, g_, rd, device=dev) * 0.1).to(bf)
+                vv = torch.randn(n, RH, rv, device=dev).to(bf)
+                dec = torch.rand(n, RH, rd, device=dev) * 0.1 + 0.9
+                beta = None
+                io = n * (2 * g_ * rd + RH * rv) * 2 + n * RH * rd * 4
+            st = rc.states["rec"]
+            row("linear_scan %s, %d x %d tokens" % (form, NB, cnt), "",
+                lambda: sk.linear_scan(qq, kk, vv, dec, beta, st, bt),
+                io + n * RH * rv * 4 + 2 * NB * RH * rd * rv * 4,
+                0.0)
+            rc.end_step()
+            del rc
+    # ---- recurrence prologue / epilogue
+    rc = PagedStateCache([], {"conv": (3, 2 * RG * rd + RH * rv)}, B,
+                         B * (S + 64), dtype=bf, device=dev)
+    bt = rc.begin_ragged(list(range(B)), [S] * B)
+    C = 2 * RG * rd + RH * rv
+    pj = torch.randn(T, C + RH * rv + 2 * RH, device=dev).to(bf)
+    cw = torch.randn(C, 4, device=dev).to(bf)
+    al, db = torch.zeros(RH, device=dev), torch.zeros(RH, device=dev)
+    row("delta_prep (conv+silu, unit q/k, gates; fp32 out)", "norm_conv",
+        lambda: sk.delta_prep(pj, bt, cw, rc.states["conv"], al, db, RG, RH,
+                              rd, rv), T * C * 6)
+    rc.end_step()
+    o32 = torch.randn(T, RH, rv, device=dev)
+    gate = torch.randn(T, RH * rv, device=dev).to(bf)
+    nw = torch.ones(rv, device=dev)
+    row("head_norm_gate (fp32 in, bf16 gate and out)", "rms_norm",
+        lambda: sk.head_norm_gate(o32, nw, gate, 1e-6, bf), T * RH * rv * 8)
+    # ---- activations
+    gu = torch.randn(T, 2 * F, device=dev).to(bf)
+    row("glu gelu_tanh", "swiglu", lambda: sk.glu(gu, 1), T * F * 6)
+    row("glu silu", "swiglu", lambda: sk.glu(gu, 0), T * F * 6)
+    zf = torch.randn(T, F, device=dev).to(bf)
+    up = torch.randn(T, F, device=dev).to(bf)
+    row("swiglu (llama)", "", lambda: swiglu(zf, up), T * F * 6)
+    return out
+
+
+def run_lolulorn(sizes=("s", "m", "l"), kernels=True):
+    dev = torch.device("cuda", torch.cuda.current_device())
+    report = {}
+    for name in sizes:
+        z = dict(SIZES[name])
+        z["layers"] = 4 if name != "l" else 4
+        rec = {"size": {k: z[k] for k in z},
+               "lolulorn": _ragged_throughput(lolulorn_config(z), z, dev),
+               "fizesun": _ragged_throughput(fizesun_config(z), z, dev),
+               "llama": _llama_throughput(z, dev)}
+        if kernels:
+            rec["kernels"] = _lolulorn_kernel_rows(z, dev)
+        report[name] = rec
+        torch.cuda.empty_cache()
+    return report
+
+
 def run(sizes=("s", "m", "l"), kernels=True):
     dev = torch.device("cuda", torch.cuda.current_device())
     report = {}
@@ -264,17 +508,20 @@ def run(sizes=("s", "m", "l"), kernels=True):
     return report
 
 
-def main(sizes="s,m,l", out=None):
-    rep = run(tuple(sizes.split(",")))
+def main(sizes="s,m,l", out=None, model="fizesun"):
+    names = tuple(sizes.split(","))
+    rep = run(names) if model == "fizesun" else run_lolulorn(names)
     if out:
         with open(out, "w") as f:
             json.dump(rep, f, indent=1)
     best = rep[sizes.split(",")[-1]]
+    extra = {} if model == "fizesun" else {"lolulorn": None}
     print(json.dumps({
-        "metric": "fizesun_serving_tokens_per_s", "unit": "tokens/s",
+        "metric": "%s_serving_tokens_per_s" % model, "unit": "tokens/s",
         "dtype": "bf16", "data": "synthetic", "n_gpus": 1,
-        "value": best["fizesun"]["prefill_tok_s"], "higher_is_better": True,
-        "sizes": {k: {"fizesun": v["fizesun"], "llama": v["llama"],
+        "value": best[model]["prefill_tok_s"], "higher_is_better": True,
+        "sizes": {k: {**{m: v[m] for m in extra}, "fizesun": v["fizesun"],
+                      "llama": v["llama"],
                       "worst_kernel_distance": max(
                           (r["distance"] for r in v.get("kernels", [])
                            if r["like"]), default=None)}

@@ -266,6 +266,309 @@ __global__ __launch_bounds__(NT) void window_attn_merge_k(
   }
 }
 
+// ------------------------------------------- windowed attention, MFMA tiles
+// bf16 path for steps that bring portions of prompts. For one sequence and one
+// key/value head g the rows are (token, query head of g) pairs, token-major:
+// row m belongs to token m / rep and head g*rep + m % rep, so the heads that
+// share keys sit in one [count*rep, dim] x [dim, keys] product. A workgroup of
+// 4 waves owns 128 rows (32 per wave) and walks the key steps (32 keys each)
+// that any of its rows can see: the steps that hold kept first tokens, then
+// the steps from the earliest window start to the last row's own position.
+//   S^T[key, row] = mfma(A = K tile from LDS, B = Q fragments in registers)
+//   mask (causal, window, kept tokens), online softmax per row (fp32)
+//   O^T[d, row]  += mfma(A = V^T tile from LDS, B = P fragments)
+// The weights stay 32-bit through the second product: P goes in as a bf16
+// head plus a bf16 remainder (two MFMAs), which carries 16 bits of mantissa.
+// mfma_f32_32x32x16_bf16 layouts: A row = lane&31, k = reg + 8*(lane>>5);
+// B col = lane&31, k = reg + 8*(lane>>5); C/D col = lane&31,
+// row = (reg&3) + 8*(reg>>2) + 4*(lane>>5).
+typedef short bf16x8s __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int TB_ROWS = 128;
+constexpr int TB_KEYS = 32;
+constexpr int VT_STRIDE = TB_KEYS + 8;
+constexpr float LAZY_MAX = 8.f;
+
+__device__ __forceinline__ float bf_bits2f(short b) {
+  union { unsigned u; float f; } c;
+  c.u = ((unsigned)(unsigned short)b) << 16;
+  return c.f;
+}
+
+template <int DKT_MAX, int DVB, bool PREFETCH>
+__global__ __launch_bounds__(256) void window_attn_mfma_k(
+    const short* __restrict__ q,     // [Ttok, H, dim]
+    const short* __restrict__ pool,  // rows of G*dim keys then G*vdim values
+    const int* __restrict__ work,    // [nwork][3] = (sequence, key/value head, first row)
+    const int* __restrict__ cu, const int* __restrict__ seq_start,
+    const int* __restrict__ table, int maxb, int bs, bf16* __restrict__ out,
+    float* __restrict__ part,  // [Ttok, nsplit, H, vdim + 2] when nsplit > 1
+    int H, int G, int dim, int vdim, int nsplit, float scale, int window, int keep_first) {
+  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+  constexpr int CPT = (2 * DKT_MAX + 4 * DVB + 7) / 8;  // 16-byte chunks per thread and tile
+  const int dimP = (dim + 15) & ~15;
+  const int DKT = dimP >> 4;
+  const int KSS = dimP + 8;
+  const int cpk = dimP >> 3;        // key chunks per row
+  const int cpv = (vdim + 7) >> 3;  // value chunks per row
+  const int dvb = (vdim + 31) >> 5;
+  short* Ks = reinterpret_cast<short*>(smem_raw);  // [TB_KEYS][KSS]
+  short* Vt = Ks + TB_KEYS * KSS;                  // [DVB*32][VT_STRIDE]
+  const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
+  const int hl = lane >> 5, l31 = lane & 31;
+  const int s = work[3 * blockIdx.x], g = work[3 * blockIdx.x + 1];
+  const int m0 = work[3 * blockIdx.x + 2];
+  const int split = blockIdx.y;
+  const int rep = H / G;
+  const int row_w = G * (dim + vdim);
+  const int count = cu[s + 1] - cu[s], start = seq_start[s];
+  const int rows = count * rep;
+  const int m_raw = m0 + wid * 32 + l31;
+  const int m = min(m_raw, rows - 1);
+  const int j = m / rep, h = g * rep + (m - j * rep);
+  const int t = cu[s] + j;
+  const int qpos = start + j;
+  const int j_lo = m0 / rep;
+  const int kmax = start + min(m0 + TB_ROWS - 1, rows - 1) / rep;  // inclusive
+  const int W = window > 0 ? window : 0x7fffffff;
+  const int lo_min = window > 0 ? max(0, start + j_lo - window + 1) : 0;
+  const int first_step = lo_min / TB_KEYS;
+  const int keep_steps = keep_first > 0 ? min((keep_first - 1) / TB_KEYS + 1, first_step) : 0;
+  const int nsteps = keep_steps + kmax / TB_KEYS - first_step + 1;
+  const int* tab = table + (int64_t)s * maxb;
+  const int per = (nsteps + nsplit - 1) / nsplit;
+  const int v_lo = split * per, v_hi = min(nsteps, v_lo + per);
+  float* pp = nullptr;
+  if (nsplit > 1) pp = part + (((int64_t)t * nsplit + split) * H + h) * (vdim + 2);
+  if (v_lo >= v_hi) {  // block-uniform: nothing to see in this split
+    if (m_raw < rows && hl == 0) {
+      pp[0] = -INFINITY;
+      pp[1] = 0.f;
+    }
+    return;
+  }
+  auto key0_of = [&](int v) -> int {
+    return (v < keep_steps ? v : first_step + v - keep_steps) * TB_KEYS;
+  };
+
+  const bool vec_ok = (dim & 7) == 0 && (vdim & 7) == 0;
+  bf16x8s qf[DKT_MAX];
+#pragma unroll
+  for (int i = 0; i < DKT_MAX; ++i) {
+    if (i < DKT) {
+      const int d0 = 16 * i + 8 * hl;
+      const short* src = q + ((int64_t)t * H + h) * dim + d0;
+      if (vec_ok && d0 + 8 <= dim) {
+        qf[i] = *reinterpret_cast<const bf16x8s*>(src);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) qf[i][e] = d0 + e < dim ? src[e] : (short)0;
+      }
+    }
+  }
+  f32x16 oacc[DVB];
+#pragma unroll
+  for (int db = 0; db < DVB; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
+  float mrun = -INFINITY, lrun = 0.f;
+
+  // Staging: chunk c of a tile is (8 values from 8*(c>>5), key c&31):
+  // neighbouring lanes take neighbouring keys, so the transposed writes of a
+  // value chunk fall into one LDS row. Every chunk of a thread belongs to the
+  // same key (256 is a multiple of 32), so the thread resolves ONE pool row
+  // per tile through the block table, a step ahead of the loads.
+  auto row_of = [&](int k0) -> int64_t {
+    const int p = k0 + (tid & 31);
+    return p <= kmax ? (int64_t)tab[p / bs] * bs + p % bs : (int64_t)-1;
+  };
+  auto fetch_one = [&](int i, int64_t row) -> bf16x8s {
+    const int c = tid + i * 256;
+    bf16x8s v;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = 0;
+    if (c < TB_KEYS * (cpk + cpv) && row >= 0) {
+      const int ch = c >> 5;
+      const bool is_k = ch < cpk;
+      const int d0 = is_k ? ch * 8 : (ch - cpk) * 8;
+      const int lim = is_k ? dim : vdim;
+      const short* src = pool + row * row_w + (is_k ? g * dim : G * dim + g * vdim) + d0;
+      if (vec_ok && d0 + 8 <= lim) {
+        v = *reinterpret_cast<const bf16x8s*>(src);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (d0 + e < lim) v[e] = src[e];
+      }
+    }
+    return v;
+  };
+  auto stash_one = [&](int i, const bf16x8s& v) {
+    const int c = tid + i * 256;
+    if (c < TB_KEYS * (cpk + cpv)) {
+      const int ch = c >> 5, key = c & 31;
+      if (ch < cpk) {
+        *reinterpret_cast<bf16x8s*>(Ks + key * KSS + ch * 8) = v;
+      } else {
+        const int d0 = (ch - cpk) * 8;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) Vt[(d0 + e) * VT_STRIDE + key] = v[e];
+      }
+    }
+  };
+  bf16x8s pre[PREFETCH ? CPT : 1];
+  auto fetch = [&](int64_t row) {
+#pragma unroll
+    for (int i = 0; i < CPT; ++i)
+      if (PREFETCH) pre[i] = fetch_one(i, row);
+  };
+  auto stash = [&](int64_t row) {
+    if (PREFETCH) {
+#pragma unroll
+      for (int i = 0; i < CPT; ++i) stash_one(i, pre[i]);
+    } else {
+#pragma unroll 1
+      for (int i = 0; i < CPT; i += 4) {
+        bf16x8s v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = fetch_one(i + u, row);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) stash_one(i + u, v[u]);
+      }
+    }
+  };
+
+  int64_t row_next = row_of(key0_of(v_lo));
+  if (PREFETCH) {
+    fetch(row_next);
+    row_next = v_lo + 1 < v_hi ? row_of(key0_of(v_lo + 1)) : (int64_t)-1;
+  }
+  for (int v = v_lo; v < v_hi; ++v) {
+    const int k0 = key0_of(v);
+    __syncthreads();
+    stash(row_next);  // without PREFETCH: fetches tile v itself
+    __syncthreads();
+    if (PREFETCH) {
+      if (v + 1 < v_hi) fetch(row_next);
+      row_next = v + 2 < v_hi ? row_of(key0_of(v + 2)) : (int64_t)-1;
+    } else {
+      row_next = v + 1 < v_hi ? row_of(key0_of(v + 1)) : (int64_t)-1;
+    }
+    f32x16 st;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) st[r] = 0.f;
+#pragma unroll
+    for (int i = 0; i < DKT_MAX; ++i) {
+      if (i < DKT) {
+        const bf16x8s kf =
+            *reinterpret_cast<const bf16x8s*>(Ks + l31 * KSS + 16 * i + 8 * hl);
+        st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[i], st, 0, 0, 0);
+      }
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int key = k0 + (r & 3) + 8 * (r >> 2) + 4 * hl;
+      const bool see = key <= qpos && (qpos - key < W || key < keep_first);
+      const float sv = see ? st[r] * scale : -INFINITY;
+      st[r] = sv;
+      mx = fmaxf(mx, sv);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    // The running maximum follows the scores lazily: it moves only when a
+    // score exceeds it by more than LAZY_MAX (weights stay below e^LAZY_MAX,
+    // harmless in fp32), so most steps need no rescaling of the sums. A row
+    // that has seen no key yet keeps weight zero without producing inf - inf.
+    const float m_new = (mx > mrun + LAZY_MAX) ? mx : mrun;
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = __expf(mrun - m_use);
+    float psum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float pw = __expf(st[r] - m_use);
+      st[r] = pw;
+      psum += pw;
+    }
+    psum += __shfl_xor(psum, 32, 64);
+    lrun = lrun * alpha + psum;
+    if (__any(m_new != mrun)) {
+#pragma unroll
+      for (int db = 0; db < DVB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
+    }
+    mrun = m_new;
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      // B fragment of P: keys 16*ks + 8*hl + 0..7 of this lane's row; half of
+      // them sit in the partner lane (lane ^ 32)
+      bf16x8s ph, pl;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float a0 = st[i + 8 * ks], a1 = st[i + 8 * ks + 4];
+        const float recv = __shfl_xor(hl ? a0 : a1, 32, 64);
+        const float x0 = hl ? recv : a0, x1 = hl ? a1 : recv;
+        ph[i] = f2bf_bits(x0);
+        ph[i + 4] = f2bf_bits(x1);
+        pl[i] = f2bf_bits(x0 - bf_bits2f(ph[i]));
+        pl[i + 4] = f2bf_bits(x1 - bf_bits2f(ph[i + 4]));
+      }
+#pragma unroll
+      for (int db = 0; db < DVB; ++db) {
+        if (db < dvb) {
+          const bf16x8s vf = *reinterpret_cast<const bf16x8s*>(
+              Vt + (32 * db + l31) * VT_STRIDE + 16 * ks + 8 * hl);
+          oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, ph, oacc[db], 0, 0, 0);
+          oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pl, oacc[db], 0, 0, 0);
+        }
+      }
+    }
+  }
+  if (m_raw < rows) {
+    if (nsplit > 1) {
+      if (hl == 0) {
+        pp[0] = mrun;
+        pp[1] = lrun;
+      }
+#pragma unroll
+      for (int db = 0; db < DVB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int d = 32 * db + (r & 3) + 8 * (r >> 2) + 4 * hl;
+          if (d < vdim) pp[2 + d] = oacc[db][r];
+        }
+    } else {
+      const float inv = 1.f / lrun;
+      bf16* o = out + ((int64_t)t * H + h) * vdim;
+#pragma unroll
+      for (int db = 0; db < DVB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int d = 32 * db + (r & 3) + 8 * (r >> 2) + 4 * hl;
+          if (d < vdim) o[d] = __float2bfloat16(oacc[db][r] * inv);
+        }
+    }
+  }
+}
+
+template <int DKT_MAX, int DVB, bool PREFETCH>
+int launch_window_attn_mfma(const void* q, const void* pool, const int* work, int nwork,
+                            const int* cu, const int* seq_start, const int* table, int maxb,
+                            int bs, void* out, float* part, int Ttok, int H, int G, int dim,
+                            int vdim, int nsplit, float scale, int window, int keep_first,
+                            hipStream_t s) {
+  const int dimP = (dim + 15) & ~15;
+  const size_t lds = (size_t)TB_KEYS * (dimP + 8) * 2 + (size_t)DVB * 32 * VT_STRIDE * 2;
+  auto kern = window_attn_mfma_k<DKT_MAX, DVB, PREFETCH>;
+  kern<<<dim3(nwork, nsplit), 256, lds, s>>>((const short*)q, (const short*)pool, work, cu,
+                                             seq_start, table, maxb, bs, (bf16*)out, part, H, G,
+                                             dim, vdim, nsplit, scale, window, keep_first);
+  if (nsplit > 1)
+    window_attn_merge_k<bf16><<<dim3(Ttok, H), NT, 0, s>>>(part, (bf16*)out, H, vdim, nsplit);
+  return (int)hipGetLastError();
+}
+
 // -------------------------------------------------- delta-rule prologue
 // proj row = [ q (G x dim) | k (G x dim) | v (H x vdim) | gate | b (H) | a (H) ].
 // One block per token: causal convolution + SiLU over the q|k|v channels
@@ -373,15 +676,25 @@ __global__ void sigmoid_pow_k(const T* __restrict__ z, const float* __restrict__
 // rows beyond dim stay zero); a block of NT threads owns NT / SCAN_R columns of
 // one head of one sequence and walks the sequence's tokens in order:
 //   S *= decay; d = S^T k; u = DELTA ? beta * (v - d) : v; S += k u; o = S^T q.
-// Sums over rows go lane-local first, then across the SCAN_R lanes in a fixed
-// order, so a result does not depend on where a sequence was cut. The next
-// token's operands are loaded while the current one is computed.
+// Sums over rows go lane-local first, then across the SCAN_R lanes by DPP
+// swaps in a fixed order, so a result does not depend on where a sequence was
+// cut. The operands of CT tokens at a time are staged through LDS (widened to
+// float, q scaled), double-buffered: the next chunk's global loads are in
+// flight while the current chunk is computed, so the token-to-token chain
+// sees LDS latency only.
 constexpr int SCAN_R = 8;
 constexpr int SCAN_COLS = NT / SCAN_R;
 
+template <int CTRL>
+__device__ __forceinline__ float dpp_swap(float x) {
+  return __int_as_float(
+      __builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, true));
+}
+// sum over the 8 lanes that share a column; every lane gets the same bits
 __device__ __forceinline__ float group_sum(float x) {
-#pragma unroll
-  for (int o = 1; o < SCAN_R; o <<= 1) x += __shfl_xor(x, o, 64);
+  x += dpp_swap<0xB1>(x);   // quad_perm [1,0,3,2]
+  x += dpp_swap<0x4E>(x);   // quad_perm [2,3,0,1]
+  x += dpp_swap<0x141>(x);  // row_half_mirror: the other quad of the 8
   return x;
 }
 
@@ -392,9 +705,23 @@ __global__ __launch_bounds__(NT) void linear_scan_k(
     const float* __restrict__ beta, float* __restrict__ state, const int* __restrict__ cu,
     const int* __restrict__ seq_slot, float* __restrict__ out, int G, int H, int dim, int vdim,
     float q_scale) {
+  constexpr int CT = ROWS <= 8 ? 16 : 8;  // tokens per staged chunk
+  constexpr int RS = ROWS + 4;            // stride of a lane's rows: 16-byte reads, spread banks
+  constexpr int KQ = SCAN_R * RS;
+  constexpr int DP = SCAN_R * ROWS;       // padded key size
+  constexpr int ND = CHANNEL_DECAY ? DP : 0;
+  constexpr int NE = 2 * DP + ND + SCAN_COLS + 2;  // staged values per token
+  constexpr int EPT = (CT * NE + NT - 1) / NT;
+  __shared__ __attribute__((aligned(16))) float sK[2][CT][KQ];
+  __shared__ __attribute__((aligned(16))) float sQ[2][CT][KQ];
+  __shared__ __attribute__((aligned(16))) float sD[2][CT][CHANNEL_DECAY ? KQ : 4];
+  __shared__ float sV[2][CT][SCAN_COLS];
+  __shared__ float sB[2][CT][2];  // beta, per-head decay
   const int s = blockIdx.x, h = blockIdx.y;
   const int r = threadIdx.x % SCAN_R;
-  const int col = blockIdx.z * SCAN_COLS + threadIdx.x / SCAN_R;
+  const int cl = threadIdx.x / SCAN_R;
+  const int col0 = blockIdx.z * SCAN_COLS;
+  const int col = col0 + cl;
   const bool live = col < vdim;
   const int cc = live ? col : vdim - 1;  // idle lanes shadow the last column
   const int g = h / (H / G);
@@ -403,60 +730,117 @@ __global__ __launch_bounds__(NT) void linear_scan_k(
   float S[ROWS];
 #pragma unroll
   for (int i = 0; i < ROWS; ++i) S[i] = r0 + i < dim ? Sg[(int64_t)(r0 + i) * vdim] : 0.f;
-  const int t0 = cu[s], t1 = cu[s + 1];
-  float kn[ROWS], qn[ROWS], dn[CHANNEL_DECAY ? ROWS : 1], vn = 0.f, bn = 1.f;
-  auto fetch = [&](int t) {
-    const T* kp = k + (int64_t)t * ld_k + g * dim + r0;
-    const T* qp = q + (int64_t)t * ld_q + g * dim + r0;
-#pragma unroll
-    for (int i = 0; i < ROWS; ++i) {
-      const bool in = r0 + i < dim;
-      kn[i] = in ? ld(kp + i) : 0.f;
-      qn[i] = in ? ld(qp + i) * q_scale : 0.f;
-    }
+  const int t0 = cu[s], n = cu[s + 1] - t0;
+  const int nchunks = (n + CT - 1) / CT;
+
+  auto load_elem = [&](int t, int e) -> float {
+    if (e < DP) return e < dim ? ld(k + (int64_t)t * ld_k + g * dim + e) : 0.f;
+    e -= DP;
+    if (e < DP) return e < dim ? ld(q + (int64_t)t * ld_q + g * dim + e) * q_scale : 0.f;
+    e -= DP;
     if (CHANNEL_DECAY) {
-      const float* dp = decay + ((int64_t)t * H + h) * dim + r0;
-#pragma unroll
-      for (int i = 0; i < ROWS; ++i) dn[i] = r0 + i < dim ? dp[i] : 0.f;
-    } else {
-      dn[0] = decay[(int64_t)t * H + h];
+      if (e < DP) return e < dim ? decay[((int64_t)t * H + h) * dim + e] : 0.f;
+      e -= DP;
     }
-    vn = ld(v + (int64_t)t * ld_v + h * vdim + cc);
-    if (DELTA) bn = beta[(int64_t)t * H + h];
+    if (e < SCAN_COLS)
+      return col0 + e < vdim ? ld(v + (int64_t)t * ld_v + h * vdim + col0 + e) : 0.f;
+    if (e == SCAN_COLS) return DELTA ? beta[(int64_t)t * H + h] : 1.f;
+    return CHANNEL_DECAY ? 1.f : decay[(int64_t)t * H + h];
   };
-  if (t0 < t1) fetch(t0);
-  for (int t = t0; t < t1; ++t) {
-    float kc[ROWS], qc[ROWS], dc[CHANNEL_DECAY ? ROWS : 1];
-#pragma unroll
-    for (int i = 0; i < ROWS; ++i) {
-      kc[i] = kn[i];
-      qc[i] = qn[i];
+  auto store_elem = [&](int b, int tk, int e, float x) {
+    if (e < DP) {
+      sK[b][tk][(e / ROWS) * RS + e % ROWS] = x;
+      return;
     }
-#pragma unroll
-    for (int i = 0; i < (CHANNEL_DECAY ? ROWS : 1); ++i) dc[i] = dn[i];
-    const float vc = vn, bc = bn;
-    if (t + 1 < t1) fetch(t + 1);
-    float u = vc;
-    if (DELTA) {
-      float d = 0.f;
-#pragma unroll
-      for (int i = 0; i < ROWS; ++i) {
-        S[i] *= CHANNEL_DECAY ? dc[i] : dc[0];
-        d += S[i] * kc[i];
+    e -= DP;
+    if (e < DP) {
+      sQ[b][tk][(e / ROWS) * RS + e % ROWS] = x;
+      return;
+    }
+    e -= DP;
+    if (CHANNEL_DECAY) {
+      if (e < DP) {
+        sD[b][tk][(e / ROWS) * RS + e % ROWS] = x;
+        return;
       }
-      u = bc * (vc - group_sum(d));
-    } else {
-#pragma unroll
-      for (int i = 0; i < ROWS; ++i) S[i] *= CHANNEL_DECAY ? dc[i] : dc[0];
+      e -= DP;
     }
-    float o = 0.f;
+    if (e < SCAN_COLS)
+      sV[b][tk][e] = x;
+    else
+      sB[b][tk][e - SCAN_COLS] = x;
+  };
+  float pre[EPT];
+  auto fetch = [&](int c) {
+    const int nt = min(CT, n - c * CT);
 #pragma unroll
-    for (int i = 0; i < ROWS; ++i) {
-      S[i] += kc[i] * u;
-      o += S[i] * qc[i];
+    for (int i = 0; i < EPT; ++i) {
+      const int f = threadIdx.x + i * NT;
+      const int tk = f / NE, e = f - tk * NE;
+      pre[i] = tk < nt ? load_elem(t0 + c * CT + tk, e) : 0.f;
     }
-    o = group_sum(o);
-    if (live && r == 0) out[((int64_t)t * H + h) * vdim + col] = o;
+  };
+  auto stash = [&](int b) {
+#pragma unroll
+    for (int i = 0; i < EPT; ++i) {
+      const int f = threadIdx.x + i * NT;
+      const int tk = f / NE, e = f - tk * NE;
+      if (tk < CT) store_elem(b, tk, e, pre[i]);
+    }
+  };
+
+  if (nchunks > 0) {
+    fetch(0);
+    stash(0);
+  }
+  __syncthreads();
+  for (int c = 0; c < nchunks; ++c) {
+    const int b = c & 1;
+    if (c + 1 < nchunks) fetch(c + 1);
+    const int nt = min(CT, n - c * CT);
+    for (int tk = 0; tk < nt; ++tk) {
+      const float4* kp = reinterpret_cast<const float4*>(&sK[b][tk][r * RS]);
+      const float4* qp = reinterpret_cast<const float4*>(&sQ[b][tk][r * RS]);
+      const float4* dp = reinterpret_cast<const float4*>(&sD[b][tk][CHANNEL_DECAY ? r * RS : 0]);
+      const float vc = sV[b][tk][cl];
+      const float bc = sB[b][tk][0], dh = sB[b][tk][1];
+      float kc[ROWS];
+#pragma unroll
+      for (int i = 0; i < ROWS / 4; ++i) {
+        const float4 x = kp[i];
+        kc[4 * i] = x.x; kc[4 * i + 1] = x.y; kc[4 * i + 2] = x.z; kc[4 * i + 3] = x.w;
+      }
+      if (CHANNEL_DECAY) {
+#pragma unroll
+        for (int i = 0; i < ROWS / 4; ++i) {
+          const float4 x = dp[i];
+          S[4 * i] *= x.x; S[4 * i + 1] *= x.y; S[4 * i + 2] *= x.z; S[4 * i + 3] *= x.w;
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < ROWS; ++i) S[i] *= dh;
+      }
+      float u = vc;
+      if (DELTA) {
+        float d = 0.f;
+#pragma unroll
+        for (int i = 0; i < ROWS; ++i) d += S[i] * kc[i];
+        u = bc * (vc - group_sum(d));
+      }
+      float o = 0.f;
+#pragma unroll
+      for (int i = 0; i < ROWS / 4; ++i) {
+        const float4 x = qp[i];
+        S[4 * i] += kc[4 * i] * u;         o += S[4 * i] * x.x;
+        S[4 * i + 1] += kc[4 * i + 1] * u; o += S[4 * i + 1] * x.y;
+        S[4 * i + 2] += kc[4 * i + 2] * u; o += S[4 * i + 2] * x.z;
+        S[4 * i + 3] += kc[4 * i + 3] * u; o += S[4 * i + 3] * x.w;
+      }
+      o = group_sum(o);
+      if (live && r == 0) out[((int64_t)(t0 + c * CT + tk) * H + h) * vdim + col] = o;
+    }
+    if (c + 1 < nchunks) stash(b ^ 1);
+    __syncthreads();
   }
   if (live) {
 #pragma unroll
@@ -523,6 +907,32 @@ int dsv_window_attn(const void* q, const void* pool, const int* tok_seq, const i
     BY_DTYPE(dt, (window_attn_merge_k<T><<<g2, NT, 0, s>>>(part, (T*)out, H, vdim, nsplit)));
   }
   return (int)hipGetLastError();
+}
+
+// 1 when the MFMA tile kernel covers these head sizes (bf16 only)
+int dsv_window_attn_mfma_ok(int dim, int vdim) {
+  return dim >= 1 && dim <= 256 && vdim >= 1 && vdim <= 256;
+}
+
+int dsv_window_attn_mfma_rows() { return TB_ROWS; }
+
+// work: [nwork][3] = (sequence, key/value head, first row of a tile of the
+// sequence's count * (H/G) rows for that head)
+int dsv_window_attn_mfma(const void* q, const void* pool, const int* work, int nwork,
+                         const int* cu, const int* seq_start, const int* table, int maxb, int bs,
+                         void* out, float* part, int Ttok, int H, int G, int dim, int vdim,
+                         int nsplit, float scale, int window, int keep_first, hipStream_t s) {
+  if (!dsv_window_attn_mfma_ok(dim, vdim) || H % G) return -1;
+  if (nsplit < 1 || (nsplit > 1 && !part)) return -3;
+  if (nwork <= 0) return 0;
+#define GO(DKT, DVB, PF)                                                                        \
+  return launch_window_attn_mfma<DKT, DVB, PF>(q, pool, work, nwork, cu, seq_start, table, maxb, \
+                                               bs, out, part, Ttok, H, G, dim, vdim, nsplit,     \
+                                               scale, window, keep_first, s)
+  if (dim <= 64 && vdim <= 64) GO(4, 2, true);
+  if (dim <= 128 && vdim <= 128) GO(8, 4, true);
+  GO(16, 8, false);
+#undef GO
 }
 
 int dsv_delta_prep(const void* proj, int ld_proj, const void* w, void* state,

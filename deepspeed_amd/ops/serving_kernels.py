@@ -455,26 +455,82 @@ def attn_prep(proj, batch, pool, q_norm_w, k_norm_w, eps, heads, kv_heads,
     return q
 
 
+def _window_tile_work(batch, kv_heads, rep, tile_rows, device):
+    """[(sequence, key/value head, first row)] over every sequence's
+    count*rep rows per key/value head, late tiles first."""
+    key = ("window_tiles", kv_heads, rep, tile_rows)
+    if key not in batch.extra:
+        import numpy as np
+        seqs, firsts, ends = [], [], []
+        for i, (st, c) in enumerate(zip(batch.starts, batch.counts)):
+            m0 = np.arange(0, c * rep, tile_rows, dtype=np.int32)
+            seqs.append(np.full(m0.shape, i, np.int32))
+            firsts.append(m0)
+            ends.append(st + (m0 + tile_rows) // rep)
+        seqs, firsts, ends = (np.concatenate(a) for a in (seqs, firsts, ends))
+        order = np.argsort(-ends, kind="stable")
+        n = order.size
+        work = np.empty((kv_heads, n, 3), np.int32)
+        work[:, :, 0] = seqs[order]
+        work[:, :, 1] = np.arange(kv_heads, dtype=np.int32)[:, None]
+        work[:, :, 2] = firsts[order]
+        work = np.ascontiguousarray(work.transpose(1, 0, 2)).reshape(-1)
+        batch.extra[key] = (torch.from_numpy(work).to(device), n * kv_heads)
+    return batch.extra[key]
+
+
+MFMA_MIN_PORTION = 8     # steps of single tokens stay with the exact kernel
+
+
 def window_attention(q, pool, batch, kv_heads, dim, vdim, scale, window=0,
                      keep_first=0, path=None):
+    """``path`` forces "mfma" or "exact" (tests); default: the bf16 tile kernel
+    when the step brings a portion of a prompt, the exact kernel for fp32 and
+    for steps of single tokens."""
     T, H, d = q.shape
     assert d == dim and T == batch.n_tokens and q.is_contiguous()
     assert pool.shape[1] == batch.block_size and pool.is_contiguous()
-    assert q.dtype == pool.dtype
+    assert q.dtype == pool.dtype and H % kv_heads == 0
+    assert pool.shape[-1] == kv_heads * (dim + vdim)
     lib = _seq()
     dt = _dt(q)
+    reach = batch.max_ctx if window <= 0 else \
+        min(batch.max_ctx, window + keep_first)
+    out = torch.empty(T, H, vdim, dtype=q.dtype, device=q.device)
+    mfma = q.dtype == torch.bfloat16 and \
+        lib.dsv_window_attn_mfma_ok(_i(dim), _i(vdim)) == 1
+    if path is None:
+        path = "mfma" if mfma and max(batch.counts) >= MFMA_MIN_PORTION \
+            else "exact"
+    if path == "mfma":
+        assert mfma, "the MFMA kernel is bf16 with head sizes up to 256"
+        rep = H // kv_heads
+        work, n = _window_tile_work(batch, kv_heads, rep,
+                                    lib.dsv_window_attn_mfma_rows(), q.device)
+        nsplit = 1
+        if n < 128:
+            nsplit = max(1, min(32, reach // 128, 512 // n))
+        part = None
+        if nsplit > 1:
+            part = torch.empty(T, nsplit, H, vdim + 2, dtype=torch.float32,
+                               device=q.device)
+        _check(lib.dsv_window_attn_mfma(
+            _p(q), _p(pool), _p(work), _i(n), _p(batch.cu),
+            _p(batch.seq_start), _p(batch.block_table),
+            _i(batch.block_table.shape[1]), _i(batch.block_size), _p(out),
+            _p(part), _i(T), _i(H), _i(kv_heads), _i(dim), _i(vdim),
+            _i(nsplit), _f(scale), _i(window), _i(keep_first), _stream()),
+            "window_attention(mfma)")
+        return out.view(T, H * vdim)
     kc = 64
     while kc > 4 and lib.dsv_window_attn_lds(dt, dim, vdim, kc) > 60 * 1024:
         kc //= 2
     # few tokens over a long visible range (decoding): split the keys so the
     # launch still covers the chip; partial sums are merged in fp32
-    reach = batch.max_ctx if window <= 0 else \
-        min(batch.max_ctx, window + keep_first)
     nsplit = 1
     if T * kv_heads <= 128:
         nsplit = max(1, min(32, reach // (4 * kc),
                             1024 // max(1, T * kv_heads)))
-    out = torch.empty(T, H, vdim, dtype=q.dtype, device=q.device)
     part = None
     if nsplit > 1:
         part = torch.empty(T, nsplit, H, vdim + 2, dtype=torch.float32,

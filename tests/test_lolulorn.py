@@ -884,3 +884,40 @@ def test_attention_kernel_sizes_against_eager(dtype, heads, kv, dim, vdim,
         cache.end_step()
         tol = 2e-5 if dtype == torch.float32 else 2e-2
         assert (got - want).abs().max().item() < tol
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("heads,kv,dim,vdim", [
+    (8, 2, 128, 128), (6, 3, 64, 64), (5, 1, 40, 24), (4, 4, 96, 160),
+    (2, 1, 256, 256), (12, 2, 20, 6)])
+def test_mfma_tiles_match_the_exact_kernel(heads, kv, dim, vdim):
+    """The bf16 tile kernel against the exact one in all three size classes:
+    a step of unequal portions and single tokens over a scrambled block table,
+    windows that cut through tiles, kept tokens in and out of the window's
+    first step, no window at all, and decoding with split keys."""
+    from deepspeed_amd.ops import serving_kernels as sk
+    g = torch.Generator().manual_seed(heads * dim + vdim)
+    bf = torch.bfloat16
+    for held, counts, win, keep in (
+            ([0, 900, 37, 5], [200, 1, 130, 2], 150, 5),
+            ([0], [333], 40, 0), ([10, 0], [70, 300], 100, 70),
+            ([700, 650], [1, 90], 0, 0), ([1500], [1], 1000, 7),
+            ([300, 0], [9, 64], 33, 33)):
+        cache = PagedStateCache([kv * (dim + vdim)], {}, len(held), 4096,
+                                block_size=64, dtype=bf, device=DEV)
+        perm = torch.randperm(len(cache.free_blocks), generator=g).tolist()
+        cache.free_blocks = [cache.free_blocks[i] for i in perm]
+        for slot, n in enumerate(held):
+            cache.reset_slot(slot)
+            cache.lens[slot] = n
+        b = cache.begin_ragged(list(range(len(held))), counts)
+        cache.pools[0].copy_(torch.randn(cache.pools[0].shape, generator=g))
+        T = sum(counts)
+        q = (torch.randn(T, heads, dim, generator=g) * 0.5).to(DEV, bf)
+        out = {}
+        for path in ("mfma", "exact"):
+            out[path] = sk.window_attention(q, cache.pools[0], b, kv, dim,
+                                            vdim, 0.2, win, keep,
+                                            path=path).float().cpu()
+        cache.end_step()
+        assert (out["mfma"] - out["exact"]).abs().max().item() < 2e-2
