@@ -674,7 +674,9 @@ __global__ void sigmoid_pow_k(const T* __restrict__ z, const float* __restrict__
 // both forms, so the work is split by column: SCAN_R lanes share a column,
 // each holding ROWS consecutive rows of it in registers (dim <= SCAN_R * ROWS,
 // rows beyond dim stay zero); a block of NT threads owns NT / SCAN_R columns of
-// one head of one sequence and walks the sequence's tokens in order:
+// one head of one sequence and walks the sequence's tokens in order (few rows
+// per lane and many lanes: the chain from token to token is short, and two
+// or more waves per SIMD fill each other's issue gaps):
 //   S *= decay; d = S^T k; u = DELTA ? beta * (v - d) : v; S += k u; o = S^T q.
 // Sums over rows go lane-local first, then across the SCAN_R lanes by DPP
 // swaps in a fixed order, so a result does not depend on where a sequence was
@@ -682,7 +684,7 @@ __global__ void sigmoid_pow_k(const T* __restrict__ z, const float* __restrict__
 // float, q scaled), double-buffered: the next chunk's global loads are in
 // flight while the current chunk is computed, so the token-to-token chain
 // sees LDS latency only.
-constexpr int SCAN_R = 8;
+constexpr int SCAN_R = 16;
 constexpr int SCAN_COLS = NT / SCAN_R;
 
 template <int CTRL>
@@ -690,11 +692,46 @@ __device__ __forceinline__ float dpp_swap(float x) {
   return __int_as_float(
       __builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, true));
 }
-// sum over the 8 lanes that share a column; every lane gets the same bits
+// sum over the 16 lanes (one DPP row) that share a column; every lane gets
+// the same bits
 __device__ __forceinline__ float group_sum(float x) {
   x += dpp_swap<0xB1>(x);   // quad_perm [1,0,3,2]
   x += dpp_swap<0x4E>(x);   // quad_perm [2,3,0,1]
   x += dpp_swap<0x141>(x);  // row_half_mirror: the other quad of the 8
+  x += dpp_swap<0x140>(x);  // row_mirror: the other half of the row
+  return x;
+}
+
+// four neighbouring values p[e..e+3] widened to float, zero beyond n
+__device__ __forceinline__ bool vec4_ok(const float* p, int ld, int n) {
+  return (reinterpret_cast<uintptr_t>(p) & 15) == 0 && (ld & 3) == 0 && (n & 3) == 0;
+}
+__device__ __forceinline__ bool vec4_ok(const bf16* p, int ld, int n) {
+  return (reinterpret_cast<uintptr_t>(p) & 7) == 0 && (ld & 3) == 0 && (n & 3) == 0;
+}
+__device__ __forceinline__ float4 load4(const float* p, int e, int n, bool vec) {
+  if (vec && e + 4 <= n) return *reinterpret_cast<const float4*>(p + e);
+  float4 x;
+  x.x = e < n ? p[e] : 0.f;
+  x.y = e + 1 < n ? p[e + 1] : 0.f;
+  x.z = e + 2 < n ? p[e + 2] : 0.f;
+  x.w = e + 3 < n ? p[e + 3] : 0.f;
+  return x;
+}
+__device__ __forceinline__ float4 load4(const bf16* p, int e, int n, bool vec) {
+  float4 x;
+  if (vec && e + 4 <= n) {
+    const uint2 w = *reinterpret_cast<const uint2*>(p + e);
+    x.x = __uint_as_float(w.x << 16);
+    x.y = __uint_as_float(w.x & 0xffff0000u);
+    x.z = __uint_as_float(w.y << 16);
+    x.w = __uint_as_float(w.y & 0xffff0000u);
+    return x;
+  }
+  x.x = e < n ? ld(p + e) : 0.f;
+  x.y = e + 1 < n ? ld(p + e + 1) : 0.f;
+  x.z = e + 2 < n ? ld(p + e + 2) : 0.f;
+  x.w = e + 3 < n ? ld(p + e + 3) : 0.f;
   return x;
 }
 
@@ -705,13 +742,10 @@ __global__ __launch_bounds__(NT) void linear_scan_k(
     const float* __restrict__ beta, float* __restrict__ state, const int* __restrict__ cu,
     const int* __restrict__ seq_slot, float* __restrict__ out, int G, int H, int dim, int vdim,
     float q_scale) {
-  constexpr int CT = ROWS <= 8 ? 16 : 8;  // tokens per staged chunk
+  constexpr int CT = ROWS <= 4 ? 16 : 8;  // tokens per staged chunk
   constexpr int RS = ROWS + 4;            // stride of a lane's rows: 16-byte reads, spread banks
   constexpr int KQ = SCAN_R * RS;
   constexpr int DP = SCAN_R * ROWS;       // padded key size
-  constexpr int ND = CHANNEL_DECAY ? DP : 0;
-  constexpr int NE = 2 * DP + ND + SCAN_COLS + 2;  // staged values per token
-  constexpr int EPT = (CT * NE + NT - 1) / NT;
   __shared__ __attribute__((aligned(16))) float sK[2][CT][KQ];
   __shared__ __attribute__((aligned(16))) float sQ[2][CT][KQ];
   __shared__ __attribute__((aligned(16))) float sD[2][CT][CHANNEL_DECAY ? KQ : 4];
@@ -733,59 +767,73 @@ __global__ __launch_bounds__(NT) void linear_scan_k(
   const int t0 = cu[s], n = cu[s + 1] - t0;
   const int nchunks = (n + CT - 1) / CT;
 
-  auto load_elem = [&](int t, int e) -> float {
-    if (e < DP) return e < dim ? ld(k + (int64_t)t * ld_k + g * dim + e) : 0.f;
-    e -= DP;
-    if (e < DP) return e < dim ? ld(q + (int64_t)t * ld_q + g * dim + e) * q_scale : 0.f;
-    e -= DP;
-    if (CHANNEL_DECAY) {
-      if (e < DP) return e < dim ? decay[((int64_t)t * H + h) * dim + e] : 0.f;
-      e -= DP;
-    }
-    if (e < SCAN_COLS)
-      return col0 + e < vdim ? ld(v + (int64_t)t * ld_v + h * vdim + col0 + e) : 0.f;
-    if (e == SCAN_COLS) return DELTA ? beta[(int64_t)t * H + h] : 1.f;
-    return CHANNEL_DECAY ? 1.f : decay[(int64_t)t * H + h];
-  };
-  auto store_elem = [&](int b, int tk, int e, float x) {
-    if (e < DP) {
-      sK[b][tk][(e / ROWS) * RS + e % ROWS] = x;
-      return;
-    }
-    e -= DP;
-    if (e < DP) {
-      sQ[b][tk][(e / ROWS) * RS + e % ROWS] = x;
-      return;
-    }
-    e -= DP;
-    if (CHANNEL_DECAY) {
-      if (e < DP) {
-        sD[b][tk][(e / ROWS) * RS + e % ROWS] = x;
-        return;
-      }
-      e -= DP;
-    }
-    if (e < SCAN_COLS)
-      sV[b][tk][e] = x;
-    else
-      sB[b][tk][e - SCAN_COLS] = x;
-  };
-  float pre[EPT];
+  // Staging: a thread moves groups of four neighbouring values (one 8- or
+  // 16-byte load when the operand allows it, one 16-byte LDS store); all sizes
+  // are powers of two, so the index arithmetic is shifts and masks.
+  constexpr int V4 = DP / 4;                         // groups of four per token
+  constexpr int VPT = (CT * V4 + NT - 1) / NT;       // per thread and operand
+  constexpr int SM = SCAN_COLS + 2;                  // v columns, beta, decay
+  constexpr int SPT = (CT * SM + NT - 1) / NT;
+  const bool vec_k = vec4_ok(k, ld_k, dim), vec_q = vec4_ok(q, ld_q, dim);
+  float4 pk[VPT], pq[VPT], pd[CHANNEL_DECAY ? VPT : 1];
+  float ps[SPT];
   auto fetch = [&](int c) {
     const int nt = min(CT, n - c * CT);
+    const int tc = t0 + c * CT;
 #pragma unroll
-    for (int i = 0; i < EPT; ++i) {
+    for (int i = 0; i < VPT; ++i) {
       const int f = threadIdx.x + i * NT;
-      const int tk = f / NE, e = f - tk * NE;
-      pre[i] = tk < nt ? load_elem(t0 + c * CT + tk, e) : 0.f;
+      const int tk = f / V4, e = (f % V4) * 4;
+      const bool in = tk < nt;
+      pk[i] = in ? load4(k + (int64_t)(tc + tk) * ld_k + g * dim, e, dim, vec_k)
+                 : make_float4(0.f, 0.f, 0.f, 0.f);
+      pq[i] = in ? load4(q + (int64_t)(tc + tk) * ld_q + g * dim, e, dim, vec_q)
+                 : make_float4(0.f, 0.f, 0.f, 0.f);
+      if (CHANNEL_DECAY)
+        pd[i] = in ? load4(decay + ((int64_t)(tc + tk) * H + h) * dim, e, dim, (dim & 3) == 0)
+                   : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+#pragma unroll
+    for (int i = 0; i < SPT; ++i) {
+      const int f = threadIdx.x + i * NT;
+      const int tk = f / SM, e = f - tk * SM;
+      float x = 0.f;
+      if (tk < nt) {
+        const int t = tc + tk;
+        if (e < SCAN_COLS)
+          x = col0 + e < vdim ? ld(v + (int64_t)t * ld_v + h * vdim + col0 + e) : 0.f;
+        else if (e == SCAN_COLS)
+          x = DELTA ? beta[(int64_t)t * H + h] : 1.f;
+        else
+          x = CHANNEL_DECAY ? 1.f : decay[(int64_t)t * H + h];
+      }
+      ps[i] = x;
     }
   };
   auto stash = [&](int b) {
 #pragma unroll
-    for (int i = 0; i < EPT; ++i) {
+    for (int i = 0; i < VPT; ++i) {
       const int f = threadIdx.x + i * NT;
-      const int tk = f / NE, e = f - tk * NE;
-      if (tk < CT) store_elem(b, tk, e, pre[i]);
+      const int tk = f / V4, e = (f % V4) * 4;
+      if (tk < CT) {
+        const int at = (e / ROWS) * RS + e % ROWS;
+        float4 x = pq[i];
+        x.x *= q_scale; x.y *= q_scale; x.z *= q_scale; x.w *= q_scale;
+        *reinterpret_cast<float4*>(&sK[b][tk][at]) = pk[i];
+        *reinterpret_cast<float4*>(&sQ[b][tk][at]) = x;
+        if (CHANNEL_DECAY) *reinterpret_cast<float4*>(&sD[b][tk][at]) = pd[i];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < SPT; ++i) {
+      const int f = threadIdx.x + i * NT;
+      const int tk = f / SM, e = f - tk * SM;
+      if (tk < CT) {
+        if (e < SCAN_COLS)
+          sV[b][tk][e] = ps[i];
+        else
+          sB[b][tk][e - SCAN_COLS] = ps[i];
+      }
     }
   };
 
@@ -798,45 +846,64 @@ __global__ __launch_bounds__(NT) void linear_scan_k(
     const int b = c & 1;
     if (c + 1 < nchunks) fetch(c + 1);
     const int nt = min(CT, n - c * CT);
-    for (int tk = 0; tk < nt; ++tk) {
+    // the operands at the head of a token's chain (k, decay) are read from
+    // LDS one token ahead; sums run as four interleaved partial sums so that
+    // a single wave per SIMD still has independent work in flight
+    float kn[ROWS], dn[CHANNEL_DECAY ? ROWS : 1];
+    auto head = [&](int tk) {
       const float4* kp = reinterpret_cast<const float4*>(&sK[b][tk][r * RS]);
+#pragma unroll
+      for (int i = 0; i < ROWS / 4; ++i) {
+        const float4 x = kp[i];
+        kn[4 * i] = x.x; kn[4 * i + 1] = x.y; kn[4 * i + 2] = x.z; kn[4 * i + 3] = x.w;
+      }
+      if (CHANNEL_DECAY) {
+        const float4* dp = reinterpret_cast<const float4*>(&sD[b][tk][r * RS]);
+#pragma unroll
+        for (int i = 0; i < ROWS / 4; ++i) {
+          const float4 x = dp[i];
+          dn[4 * i] = x.x; dn[4 * i + 1] = x.y; dn[4 * i + 2] = x.z; dn[(4 * i + 3) % (CHANNEL_DECAY ? ROWS : 1)] = x.w;
+        }
+      }
+    };
+    head(0);
+    for (int tk = 0; tk < nt; ++tk) {
       const float4* qp = reinterpret_cast<const float4*>(&sQ[b][tk][r * RS]);
-      const float4* dp = reinterpret_cast<const float4*>(&sD[b][tk][CHANNEL_DECAY ? r * RS : 0]);
       const float vc = sV[b][tk][cl];
       const float bc = sB[b][tk][0], dh = sB[b][tk][1];
       float kc[ROWS];
 #pragma unroll
-      for (int i = 0; i < ROWS / 4; ++i) {
-        const float4 x = kp[i];
-        kc[4 * i] = x.x; kc[4 * i + 1] = x.y; kc[4 * i + 2] = x.z; kc[4 * i + 3] = x.w;
-      }
+      for (int i = 0; i < ROWS; ++i) kc[i] = kn[i];
       if (CHANNEL_DECAY) {
 #pragma unroll
-        for (int i = 0; i < ROWS / 4; ++i) {
-          const float4 x = dp[i];
-          S[4 * i] *= x.x; S[4 * i + 1] *= x.y; S[4 * i + 2] *= x.z; S[4 * i + 3] *= x.w;
-        }
+        for (int i = 0; i < ROWS; ++i) S[i] *= dn[i % (CHANNEL_DECAY ? ROWS : 1)];
       } else {
 #pragma unroll
         for (int i = 0; i < ROWS; ++i) S[i] *= dh;
       }
+      if (tk + 1 < nt) head(tk + 1);
       float u = vc;
       if (DELTA) {
-        float d = 0.f;
+        float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
 #pragma unroll
-        for (int i = 0; i < ROWS; ++i) d += S[i] * kc[i];
-        u = bc * (vc - group_sum(d));
+        for (int i = 0; i < ROWS; i += 4) {
+          d0 += S[i] * kc[i];
+          d1 += S[i + 1] * kc[i + 1];
+          d2 += S[i + 2] * kc[i + 2];
+          d3 += S[i + 3] * kc[i + 3];
+        }
+        u = bc * (vc - group_sum((d0 + d1) + (d2 + d3)));
       }
-      float o = 0.f;
+      float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
 #pragma unroll
       for (int i = 0; i < ROWS / 4; ++i) {
         const float4 x = qp[i];
-        S[4 * i] += kc[4 * i] * u;         o += S[4 * i] * x.x;
-        S[4 * i + 1] += kc[4 * i + 1] * u; o += S[4 * i + 1] * x.y;
-        S[4 * i + 2] += kc[4 * i + 2] * u; o += S[4 * i + 2] * x.z;
-        S[4 * i + 3] += kc[4 * i + 3] * u; o += S[4 * i + 3] * x.w;
+        S[4 * i] += kc[4 * i] * u;         o0 += S[4 * i] * x.x;
+        S[4 * i + 1] += kc[4 * i + 1] * u; o1 += S[4 * i + 1] * x.y;
+        S[4 * i + 2] += kc[4 * i + 2] * u; o2 += S[4 * i + 2] * x.z;
+        S[4 * i + 3] += kc[4 * i + 3] * u; o3 += S[4 * i + 3] * x.w;
       }
-      o = group_sum(o);
+      const float o = group_sum((o0 + o1) + (o2 + o3));
       if (live && r == 0) out[((int64_t)(t0 + c * CT + tk) * H + h) * vdim + col] = o;
     }
     if (c + 1 < nchunks) stash(b ^ 1);
@@ -966,7 +1033,7 @@ int dsv_sigmoid_pow(const void* z, const float* bias, float* out, int dt, int64_
 }
 
 // largest head size of keys the scan covers
-int dsv_linear_scan_max_dim() { return SCAN_R * 32; }
+int dsv_linear_scan_max_dim() { return SCAN_R * 16; }
 
 // q/k/v: dtype dt with row strides in elements; decay [T, H] (channel_decay 0)
 // or [T, H, dim]; beta [T, H] or null (plain form).
@@ -985,8 +1052,7 @@ int dsv_linear_scan(const void* q, int ld_q, const void* k, int ld_k, const void
   do {                                            \
     if (dim <= SCAN_R * 4) SCAN(4, DELTA, CD);    \
     else if (dim <= SCAN_R * 8) SCAN(8, DELTA, CD);   \
-    else if (dim <= SCAN_R * 16) SCAN(16, DELTA, CD); \
-    else SCAN(32, DELTA, CD);                     \
+    else SCAN(16, DELTA, CD);                     \
   } while (0)
   if (beta && channel_decay) SCAN_BY_ROWS(true, true);
   else if (beta) SCAN_BY_ROWS(true, false);

@@ -479,14 +479,11 @@ def _window_tile_work(batch, kv_heads, rep, tile_rows, device):
     return batch.extra[key]
 
 
-MFMA_MIN_PORTION = 8     # steps of single tokens stay with the exact kernel
-
-
 def window_attention(q, pool, batch, kv_heads, dim, vdim, scale, window=0,
                      keep_first=0, path=None):
-    """``path`` forces "mfma" or "exact" (tests); default: the bf16 tile kernel
-    when the step brings a portion of a prompt, the exact kernel for fp32 and
-    for steps of single tokens."""
+    """``path`` forces "mfma" or "exact" (tests); default: the tile kernel for
+    bf16 at head sizes it covers (prompt portions and, with split keys, single
+    tokens), the exact kernel otherwise (fp32)."""
     T, H, d = q.shape
     assert d == dim and T == batch.n_tokens and q.is_contiguous()
     assert pool.shape[1] == batch.block_size and pool.is_contiguous()
@@ -500,16 +497,17 @@ def window_attention(q, pool, batch, kv_heads, dim, vdim, scale, window=0,
     mfma = q.dtype == torch.bfloat16 and \
         lib.dsv_window_attn_mfma_ok(_i(dim), _i(vdim)) == 1
     if path is None:
-        path = "mfma" if mfma and max(batch.counts) >= MFMA_MIN_PORTION \
-            else "exact"
+        path = "mfma" if mfma else "exact"
     if path == "mfma":
         assert mfma, "the MFMA kernel is bf16 with head sizes up to 256"
         rep = H // kv_heads
         work, n = _window_tile_work(batch, kv_heads, rep,
                                     lib.dsv_window_attn_mfma_rows(), q.device)
+        # few tiles over long visible ranges (decoding): split the keys so
+        # the launch still covers the chip; partial sums are merged in fp32
         nsplit = 1
-        if n < 128:
-            nsplit = max(1, min(32, reach // 128, 512 // n))
+        if n < 256:
+            nsplit = max(1, min(32, reach // 64, 1024 // n))
         part = None
         if nsplit > 1:
             part = torch.empty(T, nsplit, H, vdim + 2, dtype=torch.float32,
