@@ -78,6 +78,76 @@ __global__ __launch_bounds__(NT) void attn_prep_k(
   for (int i = threadIdx.x; i < nv; i += NT) row[nk + i] = pk[nk + i];
 }
 
+// The same with eight values per thread and the projection kept in registers
+// between the two passes (sizes that are multiples of 8, rows of up to
+// 8 * NT * PREP_G values).
+constexpr int PREP_G = 4;
+
+template <typename T>
+__device__ __forceinline__ void norm_rotate_row(
+    const T* __restrict__ in, int n, const float* __restrict__ w, int dim, int rot_dims,
+    const float* __restrict__ cs, const float* __restrict__ sn, T* __restrict__ out, float eps,
+    float* red) {
+  float x[PREP_G][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < PREP_G; ++i) {
+    const int at = (threadIdx.x + i * NT) * 8;
+    if (at < n) {
+      load8(in + at, x[i]);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += x[i][e] * x[i][e];
+    }
+  }
+  const float r = rsqrtf(block_sum(ss, red) / (float)n + eps);
+#pragma unroll
+  for (int i = 0; i < PREP_G; ++i) {
+    const int at = (threadIdx.x + i * NT) * 8;
+    if (at < n) {
+      float wv[8];
+      load8(w + at, wv);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) x[i][e] *= r * wv[e];
+      const int c0 = at % dim;
+#pragma unroll
+      for (int e = 0; e < 8; e += 2) {
+        if (c0 + e < rot_dims) {
+          const float co = cs[(c0 + e) >> 1], si = sn[(c0 + e) >> 1];
+          const float a = x[i][e], b = x[i][e + 1];
+          x[i][e] = a * co - b * si;
+          x[i][e + 1] = b * co + a * si;
+        }
+      }
+      store8(out + at, x[i]);
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(NT) void attn_prep_vec_k(
+    const T* __restrict__ proj, int ld_proj, const float* __restrict__ wq,
+    const float* __restrict__ wk, const int* __restrict__ tok_pos,
+    const int* __restrict__ tok_row, const float* __restrict__ cosT,
+    const float* __restrict__ sinT, T* __restrict__ pool, T* __restrict__ q_out, int H, int G,
+    int dim, int vdim, int rot_dims, int own_kv, float eps) {
+  __shared__ float red[NT / 64];
+  const int t = blockIdx.x;
+  const T* p = proj + (int64_t)t * ld_proj;
+  const int nq = H * dim, nk = G * dim, nv = G * vdim;
+  const int half = rot_dims >> 1;
+  const float* cs = cosT + (int64_t)tok_pos[t] * half;
+  const float* sn = sinT + (int64_t)tok_pos[t] * half;
+  norm_rotate_row(p, nq, wq, dim, rot_dims, cs, sn, q_out + (int64_t)t * nq, eps, red);
+  if (!own_kv) return;
+  T* row = pool + (int64_t)tok_row[t] * (nk + nv);
+  norm_rotate_row(p + nq, nk, wk, dim, rot_dims, cs, sn, row, eps, red);
+  for (int at = threadIdx.x * 8; at < nv; at += NT * 8) {
+    float x[8];
+    load8(p + nq + nk + at, x);
+    store8(row + nk + at, x);
+  }
+}
+
 // ------------------------------------------------------ windowed attention
 // Exact kernel: one block per (token, key/value head, key split); the query
 // heads of that key/value head go in groups of WHG. The keys a token sees are
@@ -945,6 +1015,14 @@ int dsv_attn_prep(const void* proj, int ld_proj, const float* wq, const float* w
                   int rot_dims, int own_kv, float eps, hipStream_t s) {
   if (rot_dims < 0 || (rot_dims & 1) || rot_dims > dim || H % G) return -1;
   if (Ttok <= 0) return 0;
+  const int row_max = 8 * NT * PREP_G;
+  if (dim % 8 == 0 && vdim % 8 == 0 && ld_proj % 8 == 0 && H * dim <= row_max &&
+      G * dim <= row_max) {
+    BY_DTYPE(dt, (attn_prep_vec_k<T><<<Ttok, NT, 0, s>>>(
+                     (const T*)proj, ld_proj, wq, wk, tok_pos, tok_row, cosT, sinT, (T*)pool,
+                     (T*)q_out, H, G, dim, vdim, rot_dims, own_kv, eps)));
+    return (int)hipGetLastError();
+  }
   BY_DTYPE(dt, (attn_prep_k<T><<<Ttok, NT, 0, s>>>((const T*)proj, ld_proj, wq, wk, tok_pos,
                                                    tok_row, cosT, sinT, (T*)pool, (T*)q_out, H,
                                                    G, dim, vdim, rot_dims, own_kv, eps)));

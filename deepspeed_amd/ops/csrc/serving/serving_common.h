@@ -38,6 +38,34 @@ __device__ __forceinline__ float wave_max(float x) {
   return x;
 }
 
+// eight neighbouring values (16-byte aligned for bf16, 32 for float) widened
+// to float, and back with one rounding
+__device__ __forceinline__ void load8(const float* p, float (&x)[8]) {
+  const float4 a = *reinterpret_cast<const float4*>(p);
+  const float4 b = *reinterpret_cast<const float4*>(p + 4);
+  x[0] = a.x; x[1] = a.y; x[2] = a.z; x[3] = a.w;
+  x[4] = b.x; x[5] = b.y; x[6] = b.z; x[7] = b.w;
+}
+__device__ __forceinline__ void load8(const bf16* p, float (&x)[8]) {
+  const uint4 w = *reinterpret_cast<const uint4*>(p);
+  x[0] = __uint_as_float(w.x << 16); x[1] = __uint_as_float(w.x & 0xffff0000u);
+  x[2] = __uint_as_float(w.y << 16); x[3] = __uint_as_float(w.y & 0xffff0000u);
+  x[4] = __uint_as_float(w.z << 16); x[5] = __uint_as_float(w.z & 0xffff0000u);
+  x[6] = __uint_as_float(w.w << 16); x[7] = __uint_as_float(w.w & 0xffff0000u);
+}
+__device__ __forceinline__ void store8(float* p, const float (&x)[8]) {
+  *reinterpret_cast<float4*>(p) = make_float4(x[0], x[1], x[2], x[3]);
+  *reinterpret_cast<float4*>(p + 4) = make_float4(x[4], x[5], x[6], x[7]);
+}
+__device__ __forceinline__ void store8(bf16* p, const float (&x)[8]) {
+  uint4 w;
+  w.x = (unsigned short)f2bf_bits(x[0]) | ((unsigned)(unsigned short)f2bf_bits(x[1]) << 16);
+  w.y = (unsigned short)f2bf_bits(x[2]) | ((unsigned)(unsigned short)f2bf_bits(x[3]) << 16);
+  w.z = (unsigned short)f2bf_bits(x[4]) | ((unsigned)(unsigned short)f2bf_bits(x[5]) << 16);
+  w.w = (unsigned short)f2bf_bits(x[6]) | ((unsigned)(unsigned short)f2bf_bits(x[7]) << 16);
+  *reinterpret_cast<uint4*>(p) = w;
+}
+
 constexpr int NT = 256;  // threads per block for the row kernels
 
 // every thread gets the block total; scratch holds NT/64 floats

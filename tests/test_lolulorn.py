@@ -921,3 +921,64 @@ def test_mfma_tiles_match_the_exact_kernel(heads, kv, dim, vdim):
                                             path=path).float().cpu()
         cache.end_step()
         assert (out["mfma"] - out["exact"]).abs().max().item() < 2e-2
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads,kv,dim,vdim,dims", [(8, 2, 128, 128, 64),
+                                                     (3, 1, 40, 24, 40),
+                                                     (16, 4, 64, 8, 2),
+                                                     (2, 2, 12, 20, 6)])
+def test_attention_prologue_kernels_against_eager(dtype, heads, kv, dim, vdim,
+                                                  dims, monkeypatch):
+    """Vector path (sizes in multiples of 8) and scalar path of the prologue:
+    queries, the rows written into a scrambled pool, and a borrowing layer
+    that writes nothing."""
+    from deepspeed_amd.ops import window_attention as wa
+    from deepspeed_amd.ops.rope import rope_tables
+    g = torch.Generator().manual_seed(dim)
+    counts, held = [5, 1, 11], [0, 70, 9]
+    T = sum(counts)
+    cos, sin = rope_tables(dims, 256, 1000.0, device=DEV, scaling=2.0)
+    wq = (1 + 0.3 * torch.randn(heads * dim, generator=g)).to(DEV)
+    wk = (1 + 0.3 * torch.randn(kv * dim, generator=g)).to(DEV)
+    for own in (True, False):
+        n = heads * dim + (kv * (dim + vdim) if own else 0)
+        proj = torch.randn(T, n, generator=g).to(DEV, dtype)
+        res = {}
+        for mode in ("kernel", "eager"):
+            if mode == "eager":
+                monkeypatch.setenv("DS_AMD_SERVING_EAGER", "1")
+            cache = PagedStateCache([kv * (dim + vdim)], {}, 3, 256,
+                                    block_size=16, dtype=dtype, device=DEV)
+            cache.free_blocks = cache.free_blocks[::2] + cache.free_blocks[1::2]
+            for slot, m in enumerate(held):
+                cache.reset_slot(slot)
+                cache.lens[slot] = m
+            b = cache.begin_ragged([0, 1, 2], counts)
+            q = wa.attn_prep(proj, b, cache.pools[0], wq, wk, 1e-5, heads, kv,
+                             dim, vdim, dims, cos, sin, own)
+            res[mode] = (q.float().cpu(), cache.pools[0].float().cpu())
+            cache.end_step()
+        monkeypatch.delenv("DS_AMD_SERVING_EAGER")
+        tol = 1e-5 if dtype == torch.float32 else 4e-2
+        assert (res["kernel"][0] - res["eager"][0]).abs().max().item() < tol
+        assert (res["kernel"][1] - res["eager"][1]).abs().max().item() < tol
+        if not own:
+            assert res["kernel"][1].abs().max().item() == 0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("ff", [64, 36])
+def test_gated_activation_kernels_against_eager(dtype, ff, monkeypatch):
+    from deepspeed_amd.ops.activations import glu
+    g = torch.Generator().manual_seed(ff)
+    gu = (torch.randn(37, 2 * ff, generator=g) * 3).to(DEV, dtype)
+    for act in ("silu", "gelu_tanh"):
+        got = glu(gu, act).float().cpu()
+        monkeypatch.setenv("DS_AMD_SERVING_EAGER", "1")
+        want = glu(gu, act).float().cpu()
+        monkeypatch.delenv("DS_AMD_SERVING_EAGER")
+        tol = 1e-5 if dtype == torch.float32 else 0.1
+        assert (got - want).abs().max().item() < tol * (1 + want.abs().max().item())
