@@ -359,6 +359,7 @@ constexpr int TB_ROWS = 128;
 constexpr int TB_KEYS = 32;
 constexpr int VT_STRIDE = TB_KEYS + 8;
 constexpr float LAZY_MAX = 8.f;
+constexpr bool P_TWO = true;  // weights as bf16 head + remainder in the second product
 
 __device__ __forceinline__ float bf_bits2f(short b) {
   union { unsigned u; float f; } c;
@@ -590,7 +591,7 @@ __global__ __launch_bounds__(256) void window_attn_mfma_k(
           const bf16x8s vf = *reinterpret_cast<const bf16x8s*>(
               Vt + (32 * db + l31) * VT_STRIDE + 16 * ks + 8 * hl);
           oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, ph, oacc[db], 0, 0, 0);
-          oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pl, oacc[db], 0, 0, 0);
+          if (P_TWO) oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pl, oacc[db], 0, 0, 0);
         }
       }
     }
@@ -679,6 +680,77 @@ __global__ __launch_bounds__(NT) void delta_prep_k(
       ys[c] = y;
     else
       v_out[(int64_t)t * nv + c - 2 * nqk] = y;
+  }
+  __syncthreads();
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+  const float qscale = rsqrtf((float)dim);
+  for (int hd = wid; hd < 2 * G; hd += NT / 64) {
+    const float* y = ys + hd * dim;
+    float ss = 0.f;
+    for (int c = lane; c < dim; c += 64) ss += y[c] * y[c];
+    ss = wave_sum(ss);
+    const float inv = rsqrtf(ss + 1e-6f) * (hd < G ? qscale : 1.f);
+    float* o = hd < G ? q_out + ((int64_t)t * G + hd) * dim
+                      : k_out + ((int64_t)t * G + hd - G) * dim;
+    for (int c = lane; c < dim; c += 64) o[c] = y[c] * inv;
+  }
+  for (int h = threadIdx.x; h < H; h += NT) {
+    beta[(int64_t)t * H + h] = sigmoidf_(ld(p + C + nv + h));
+    const float dt = softplusf_(ld(p + C + nv + H + h) + dt_bias[h]);
+    decay[(int64_t)t * H + h] = expf(-expf(a_log[h]) * dt);
+  }
+}
+
+// The same with eight channels per thread (sizes in multiples of 8).
+template <typename T, int TAPS>
+__global__ __launch_bounds__(NT) void delta_prep_vec_k(
+    const T* __restrict__ proj, int ld_proj, const T* __restrict__ w,
+    const T* __restrict__ state, int64_t state_slot_stride, const int* __restrict__ cu,
+    const int* __restrict__ seq_slot, const int* __restrict__ tok_seq,
+    const int* __restrict__ tok_pos, const float* __restrict__ a_log,
+    const float* __restrict__ dt_bias, float* __restrict__ q_out, float* __restrict__ k_out,
+    float* __restrict__ v_out, float* __restrict__ beta, float* __restrict__ decay, int G, int H,
+    int dim, int vdim) {
+  extern __shared__ float ys[];  // [2*G*dim] conv outputs of q and k
+  constexpr int TAIL = TAPS - 1;
+  const int t = blockIdx.x;
+  const int s = tok_seq[t];
+  const int j = t - cu[s];
+  const int pos = tok_pos[t];
+  const int nqk = G * dim, nv = H * vdim;
+  const int C = 2 * nqk + nv;
+  const T* sl = state + (int64_t)seq_slot[s] * state_slot_stride;
+  const T* p = proj + (int64_t)t * ld_proj;
+  for (int c = threadIdx.x * 8; c < C; c += NT * 8) {
+    float wv[8 * TAPS];  // channel-major: wv[e * TAPS + tap]
+#pragma unroll
+    for (int i = 0; i < TAPS; ++i) {
+      float tmp[8];
+      load8(w + (int64_t)c * TAPS + 8 * i, tmp);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) wv[8 * i + e] = tmp[e];
+    }
+    float acc[8], x[8];
+    load8(p + c, x);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = wv[e * TAPS + TAIL] * x[e];
+#pragma unroll
+    for (int k = 1; k <= TAIL; ++k) {
+      if (pos - k >= 0) {  // block-uniform
+        if (k <= j)
+          load8(p - (int64_t)k * ld_proj + c, x);
+        else
+          load8(sl + (int64_t)(TAIL + j - k) * C + c, x);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] += wv[e * TAPS + TAIL - k] * x[e];
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = siluf_(acc[e]);
+    if (c < 2 * nqk)
+      store8(ys + c, acc);
+    else
+      store8(v_out + (int64_t)t * nv + c - 2 * nqk, acc);
   }
   __syncthreads();
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
@@ -1091,6 +1163,20 @@ int dsv_delta_prep(const void* proj, int ld_proj, const void* w, void* state,
   const int64_t lds = (int64_t)2 * G * dim * 4;
   if (lds > 64 * 1024) return -2;
   const int C = 2 * G * dim + H * vdim;
+  // the state's rows are C wide, so C % 8 keeps every 8-channel group aligned
+  const bool vec = dim % 8 == 0 && vdim % 8 == 0 && ld_proj % 8 == 0 &&
+                   state_slot_stride % 8 == 0 && (taps == 2 || taps == 4);
+#define PREP_VEC(TAPS)                                                                         \
+  BY_DTYPE(dt, (delta_prep_vec_k<T, TAPS><<<Ttok, NT, lds, s>>>(                                \
+                   (const T*)proj, ld_proj, (const T*)w, (const T*)state, state_slot_stride,   \
+                   cu, seq_slot, tok_seq, tok_pos, a_log, dt_bias, q_out, k_out, v_out, beta,  \
+                   decay, G, H, dim, vdim)))
+  if (vec && taps == 4)
+    PREP_VEC(4);
+  else if (vec && taps == 2)
+    PREP_VEC(2);
+  else
+#undef PREP_VEC
   BY_DTYPE(dt, (delta_prep_k<T><<<Ttok, NT, lds, s>>>(
                    (const T*)proj, ld_proj, (const T*)w, (const T*)state, state_slot_stride, cu,
                    seq_slot, tok_seq, tok_pos, a_log, dt_bias, q_out, k_out, v_out, beta, decay,

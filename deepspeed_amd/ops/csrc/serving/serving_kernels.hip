@@ -66,6 +66,65 @@ __global__ __launch_bounds__(NT) void layer_norm_k(
   }
 }
 
+// The same with eight columns per thread and the row kept in registers over
+// the three passes (C a multiple of 8, at most 8 * NT * LN_G).
+constexpr int LN_G = 4;
+template <typename TI, typename TO, bool ADD>
+__global__ __launch_bounds__(NT) void layer_norm_vec_k(
+    const TI* __restrict__ in, const int64_t* __restrict__ idx,
+    const float* __restrict__ w, const float* __restrict__ b, float* __restrict__ x,
+    TO* __restrict__ out, int C, float eps) {
+  __shared__ float red[NT / 64];
+  const int64_t r = blockIdx.x;
+  const TI* row = in + (idx ? idx[r] : r) * (int64_t)C;
+  float v[LN_G][8];
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < LN_G; ++i) {
+    const int c = (threadIdx.x + i * NT) * 8;
+    if (c < C) {
+      load8(row + c, v[i]);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sum += v[i][e];
+    }
+  }
+  const float mean = block_sum(sum, red) / (float)C;
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < LN_G; ++i) {
+    const int c = (threadIdx.x + i * NT) * 8;
+    if (c < C) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        v[i][e] -= mean;
+        ss += v[i][e] * v[i][e];
+      }
+    }
+  }
+  const float inv = rsqrtf(block_sum(ss, red) / (float)C + eps);
+#pragma unroll
+  for (int i = 0; i < LN_G; ++i) {
+    const int c = (threadIdx.x + i * NT) * 8;
+    if (c < C) {
+      float wv[8], bv[8];
+      load8(w + c, wv);
+      load8(b + c, bv);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[i][e] = v[i][e] * inv * wv[e] + bv[e];
+      if (ADD) {
+        float xv[8];
+        load8(x + r * C + c, xv);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[i][e] += xv[e];
+        store8(x + r * C + c, v[i]);
+        if (out) store8(out + r * C + c, v[i]);
+      } else {
+        store8(out + r * C + c, v[i]);
+      }
+    }
+  }
+}
+
 // out[r] = table[ids[r]] * scale (fp32)
 template <typename T>
 __global__ __launch_bounds__(NT) void embed_rows_k(
@@ -604,8 +663,15 @@ int dsv_layer_norm(const void* in, int in_dt, const int64_t* idx, const float* w
   if (rows <= 0) return 0;
   if (add && !x) return -1;
   if (!add && !out) return -1;
-#define LN(TI, TO, ADD)                                                                   \
-  layer_norm_k<TI, TO, ADD><<<rows, NT, 0, s>>>((const TI*)in, idx, w, b, x, (TO*)out, C, eps)
+#define LN(TI, TO, ADD)                                                                     \
+  do {                                                                                      \
+    if (C % 8 == 0 && C <= 8 * NT * LN_G)                                                   \
+      layer_norm_vec_k<TI, TO, ADD><<<rows, NT, 0, s>>>((const TI*)in, idx, w, b, x,         \
+                                                        (TO*)out, C, eps);                  \
+    else                                                                                    \
+      layer_norm_k<TI, TO, ADD><<<rows, NT, 0, s>>>((const TI*)in, idx, w, b, x, (TO*)out,   \
+                                                    C, eps);                                \
+  } while (0)
   if (add) {
     if (in_dt == 0 && out_dt == 0) LN(float, float, true);
     else if (in_dt == 0) LN(float, bf16, true);

@@ -982,3 +982,50 @@ def test_gated_activation_kernels_against_eager(dtype, ff, monkeypatch):
         monkeypatch.delenv("DS_AMD_SERVING_EAGER")
         tol = 1e-5 if dtype == torch.float32 else 0.1
         assert (got - want).abs().max().item() < tol * (1 + want.abs().max().item())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads,kv,dim,vdim,taps", [(4, 2, 128, 256, 4),
+                                                     (2, 1, 16, 8, 2),
+                                                     (3, 3, 24, 40, 3),
+                                                     (2, 2, 10, 12, 4)])
+def test_delta_prologue_kernels_against_eager(dtype, heads, kv, dim, vdim,
+                                              taps, monkeypatch):
+    """Vector path (multiples of 8, 2 or 4 taps) and scalar path: a step of
+    unequal portions continuing from carried tails, then a second step of
+    single tokens that shifts the tails."""
+    from deepspeed_amd.ops import linear_recurrence as lr
+    g = torch.Generator().manual_seed(dim + taps)
+    C = 2 * kv * dim + heads * vdim
+    n = C + heads * vdim + 2 * heads
+    w = (torch.randn(C, taps, generator=g) * 0.5).to(DEV, dtype)
+    a_log = (torch.randn(heads, generator=g) - 1).to(DEV)
+    dtb = (torch.randn(heads, generator=g) - 1).to(DEV)
+    steps = [[6, 1, 2], [1, 1, 1]]
+    projs = [torch.randn(sum(c), n, generator=g).to(DEV, dtype) for c in steps]
+    res = {}
+    for mode in ("kernel", "eager"):
+        if mode == "eager":
+            monkeypatch.setenv("DS_AMD_SERVING_EAGER", "1")
+        cache = PagedStateCache([], {"conv": (taps - 1, C)}, 3, 256,
+                                block_size=16, dtype=dtype, device=DEV)
+        gs = torch.Generator().manual_seed(5)
+        cache.states["conv"].copy_(torch.randn(cache.states["conv"].shape,
+                                               generator=gs))
+        for slot, m in enumerate([9, 30, 2]):
+            cache.lens[slot] = m
+            if m < taps - 1:         # before a sequence's start the tail is zero
+                cache.states["conv"][slot, :taps - 1 - m] = 0
+        outs = []
+        for counts, proj in zip(steps, projs):
+            b = cache.begin_ragged([0, 1, 2], counts)
+            outs += [o.float().cpu() for o in lr.delta_prep(
+                proj, b, w, cache.states["conv"], a_log, dtb, kv, heads, dim,
+                vdim)]
+            cache.end_step()
+        res[mode] = outs + [cache.states["conv"].float().cpu()]
+    monkeypatch.delenv("DS_AMD_SERVING_EAGER")
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    for a, b in zip(res["kernel"], res["eager"]):
+        assert (a - b).abs().max().item() < tol
