@@ -53,7 +53,8 @@ class LolulornConfig:
     def from_dict(cls, d: dict) -> "LolulornConfig":
         cfg = cls(vocab_size=int(d["vocab"]), width=int(d["width"]),
                   layers=list(d["layers"]), norm_eps=float(d["norm"]["eps"]),
-                  embed_scale=float(d["embedding"]["scale"]))
+                  embed_scale=float((d.get("embedding") or {})
+                                    .get("scale", 1.0)))
         cfg.validate()
         return cfg
 
@@ -80,7 +81,8 @@ class LolulornConfig:
                 raise ValueError(f"layer {i}: kv_from must name an earlier "
                                  "attention layer with rows of its own")
             a, b = spec["mixer"], self.layers[int(src)]["mixer"]
-            if any(a[k] != b[k] for k in ("kv_heads", "dim", "vdim", "rot")):
+            if any(a.get(k, a["heads"]) != b.get(k, b["heads"])
+                   for k in ("kv_heads", "dim", "vdim", "rot")):
                 raise ValueError(f"layer {i}: kv_from layer differs in shape")
 
 
@@ -94,12 +96,17 @@ class WindowAttention(nn.Module):
 
     def __init__(self, width, m: dict, eps, dtype):
         super().__init__()
-        self.heads, self.kv_heads = int(m["heads"]), int(m["kv_heads"])
-        self.dim, self.vdim = int(m["dim"]), int(m["vdim"])
-        self.rot_dims = int(m["rot"]["dims"])
-        self.rot_base = float(m["rot"]["base"])
-        self.rot_factor = float((m["rot"].get("scaling") or {})
-                                .get("factor", 1.0))
+        self.heads = int(m["heads"])
+        self.kv_heads = int(m.get("kv_heads", self.heads))
+        self.dim, self.vdim = int(m["dim"]), int(m.get("vdim", m["dim"]))
+        rot = m.get("rot") or {}
+        self.rot_dims = int(rot.get("dims", 0))
+        self.rot_base = float(rot.get("base", 10000.0))
+        self.rot_factor = float((rot.get("scaling") or {}).get("factor", 1.0))
+        if self.heads % self.kv_heads or self.rot_dims % 2 or \
+                self.rot_dims > self.dim:
+            raise ValueError("attention: heads must be a multiple of kv_heads "
+                             "and rot.dims even and at most dim")
         self.scale = float(m["scale"])
         mask = m.get("mask") or {}
         self.window = int(mask.get("size", 0))
@@ -138,9 +145,12 @@ class GatedDeltaRule(nn.Module):
 
     def __init__(self, width, m: dict, eps, dtype):
         super().__init__()
-        self.heads, self.kv_heads = int(m["heads"]), int(m["kv_heads"])
+        self.heads = int(m["heads"])
+        self.kv_heads = int(m.get("kv_heads", self.heads))
         self.dim, self.vdim, self.taps = int(m["dim"]), int(m["vdim"]), \
-            int(m["conv"])
+            int(m.get("conv", 1))
+        if self.heads % self.kv_heads or self.taps < 1:
+            raise ValueError("delta: heads must be a multiple of kv_heads")
         self.eps = eps
         nqk, nv = self.kv_heads * self.dim, self.heads * self.vdim
         self.conv_channels = 2 * nqk + nv
