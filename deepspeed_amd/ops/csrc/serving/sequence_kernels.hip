@@ -361,14 +361,22 @@ constexpr int VT_STRIDE = TB_KEYS + 8;
 constexpr float LAZY_MAX = 8.f;
 constexpr bool P_TWO = true;  // weights as bf16 head + remainder in the second product
 
+// round-to-nearest-even through the native conversion (one packed
+// instruction per two values on gfx950)
+__device__ __forceinline__ short f2bf_native(float f) {
+  const __bf16 b = static_cast<__bf16>(f);
+  return __builtin_bit_cast(short, b);
+}
 __device__ __forceinline__ float bf_bits2f(short b) {
   union { unsigned u; float f; } c;
   c.u = ((unsigned)(unsigned short)b) << 16;
   return c.f;
 }
 
+// two workgroups per CU for the classes whose registers allow it: one hides
+// the other's barriers and softmax behind its products
 template <int DKT_MAX, int DVB, bool PREFETCH>
-__global__ __launch_bounds__(256) void window_attn_mfma_k(
+__global__ __launch_bounds__(256, (DKT_MAX <= 8 ? 2 : 1)) void window_attn_mfma_k(
     const short* __restrict__ q,     // [Ttok, H, dim]
     const short* __restrict__ pool,  // rows of G*dim keys then G*vdim values
     const int* __restrict__ work,    // [nwork][3] = (sequence, key/value head, first row)
@@ -384,8 +392,11 @@ __global__ __launch_bounds__(256) void window_attn_mfma_k(
   const int cpk = dimP >> 3;        // key chunks per row
   const int cpv = (vdim + 7) >> 3;  // value chunks per row
   const int dvb = (vdim + 31) >> 5;
-  short* Ks = reinterpret_cast<short*>(smem_raw);  // [TB_KEYS][KSS]
-  short* Vt = Ks + TB_KEYS * KSS;                  // [DVB*32][VT_STRIDE]
+  // one tile = K [TB_KEYS][KSS] then V^T [DVB*32][VT_STRIDE]; with PREFETCH two
+  // tiles alternate, so a step needs one barrier and the next tile's LDS
+  // writes overlap this tile's products
+  const int tile_sz = TB_KEYS * KSS + DVB * 32 * VT_STRIDE;
+  short* tiles = reinterpret_cast<short*>(smem_raw);
   const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
   const int hl = lane >> 5, l31 = lane & 31;
   const int s = work[3 * blockIdx.x], g = work[3 * blockIdx.x + 1];
@@ -475,7 +486,8 @@ __global__ __launch_bounds__(256) void window_attn_mfma_k(
     }
     return v;
   };
-  auto stash_one = [&](int i, const bf16x8s& v) {
+  auto stash_one = [&](int i, const bf16x8s& v, short* Ks) {
+    short* Vt = Ks + TB_KEYS * KSS;
     const int c = tid + i * 256;
     if (c < TB_KEYS * (cpk + cpv)) {
       const int ch = c >> 5, key = c & 31;
@@ -494,10 +506,10 @@ __global__ __launch_bounds__(256) void window_attn_mfma_k(
     for (int i = 0; i < CPT; ++i)
       if (PREFETCH) pre[i] = fetch_one(i, row);
   };
-  auto stash = [&](int64_t row) {
+  auto stash = [&](int64_t row, short* Ks) {
     if (PREFETCH) {
 #pragma unroll
-      for (int i = 0; i < CPT; ++i) stash_one(i, pre[i]);
+      for (int i = 0; i < CPT; ++i) stash_one(i, pre[i], Ks);
     } else {
 #pragma unroll 1
       for (int i = 0; i < CPT; i += 4) {
@@ -505,27 +517,40 @@ __global__ __launch_bounds__(256) void window_attn_mfma_k(
 #pragma unroll
         for (int u = 0; u < 4; ++u) v[u] = fetch_one(i + u, row);
 #pragma unroll
-        for (int u = 0; u < 4; ++u) stash_one(i + u, v[u]);
+        for (int u = 0; u < 4; ++u) stash_one(i + u, v[u], Ks);
       }
     }
   };
 
+  // the wave's rows span these query positions (for skipping the mask on
+  // tiles that every row sees whole)
+  const int w_first = min(m0 + wid * 32, rows - 1), w_last = min(m0 + wid * 32 + 31, rows - 1);
+  const int qpos_lo = start + w_first / rep, qpos_hi = start + w_last / rep;
+
   int64_t row_next = row_of(key0_of(v_lo));
   if (PREFETCH) {
     fetch(row_next);
-    row_next = v_lo + 1 < v_hi ? row_of(key0_of(v_lo + 1)) : (int64_t)-1;
+    stash(row_next, tiles);
+    if (v_lo + 1 < v_hi) fetch(row_of(key0_of(v_lo + 1)));
+    row_next = v_lo + 2 < v_hi ? row_of(key0_of(v_lo + 2)) : (int64_t)-1;
+    __syncthreads();
   }
   for (int v = v_lo; v < v_hi; ++v) {
     const int k0 = key0_of(v);
-    __syncthreads();
-    stash(row_next);  // without PREFETCH: fetches tile v itself
-    __syncthreads();
+    short* Ks = tiles;
     if (PREFETCH) {
-      if (v + 1 < v_hi) fetch(row_next);
-      row_next = v + 2 < v_hi ? row_of(key0_of(v + 2)) : (int64_t)-1;
+      const int cur = (v - v_lo) & 1;
+      Ks = tiles + cur * tile_sz;
+      if (v + 1 < v_hi) stash(0, tiles + (cur ^ 1) * tile_sz);  // tile v + 1
+      if (v + 2 < v_hi) fetch(row_next);
+      row_next = v + 3 < v_hi ? row_of(key0_of(v + 3)) : (int64_t)-1;
     } else {
+      __syncthreads();
+      stash(row_next, tiles);  // fetches tile v itself
+      __syncthreads();
       row_next = v + 1 < v_hi ? row_of(key0_of(v + 1)) : (int64_t)-1;
     }
+    const short* Vt = Ks + TB_KEYS * KSS;
     f32x16 st;
 #pragma unroll
     for (int r = 0; r < 16; ++r) st[r] = 0.f;
@@ -538,13 +563,22 @@ __global__ __launch_bounds__(256) void window_attn_mfma_k(
       }
     }
     float mx = -INFINITY;
+    if (k0 + TB_KEYS - 1 <= qpos_lo &&
+        (qpos_hi - k0 < W || k0 + TB_KEYS - 1 < keep_first)) {  // wave-uniform
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int key = k0 + (r & 3) + 8 * (r >> 2) + 4 * hl;
-      const bool see = key <= qpos && (qpos - key < W || key < keep_first);
-      const float sv = see ? st[r] * scale : -INFINITY;
-      st[r] = sv;
-      mx = fmaxf(mx, sv);
+      for (int r = 0; r < 16; ++r) {
+        st[r] *= scale;
+        mx = fmaxf(mx, st[r]);
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int key = k0 + (r & 3) + 8 * (r >> 2) + 4 * hl;
+        const bool see = key <= qpos && (qpos - key < W || key < keep_first);
+        const float sv = see ? st[r] * scale : -INFINITY;
+        st[r] = sv;
+        mx = fmaxf(mx, sv);
+      }
     }
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     // The running maximum follows the scores lazily: it moves only when a
@@ -580,10 +614,10 @@ __global__ __launch_bounds__(256) void window_attn_mfma_k(
         const float a0 = st[i + 8 * ks], a1 = st[i + 8 * ks + 4];
         const float recv = __shfl_xor(hl ? a0 : a1, 32, 64);
         const float x0 = hl ? recv : a0, x1 = hl ? a1 : recv;
-        ph[i] = f2bf_bits(x0);
-        ph[i + 4] = f2bf_bits(x1);
-        pl[i] = f2bf_bits(x0 - bf_bits2f(ph[i]));
-        pl[i + 4] = f2bf_bits(x1 - bf_bits2f(ph[i + 4]));
+        ph[i] = f2bf_native(x0);
+        ph[i + 4] = f2bf_native(x1);
+        pl[i] = f2bf_native(x0 - bf_bits2f(ph[i]));
+        pl[i + 4] = f2bf_native(x1 - bf_bits2f(ph[i + 4]));
       }
 #pragma unroll
       for (int db = 0; db < DVB; ++db) {
@@ -595,6 +629,7 @@ __global__ __launch_bounds__(256) void window_attn_mfma_k(
         }
       }
     }
+    if (PREFETCH) __syncthreads();
   }
   if (m_raw < rows) {
     if (nsplit > 1) {
@@ -630,7 +665,8 @@ int launch_window_attn_mfma(const void* q, const void* pool, const int* work, in
                             int vdim, int nsplit, float scale, int window, int keep_first,
                             hipStream_t s) {
   const int dimP = (dim + 15) & ~15;
-  const size_t lds = (size_t)TB_KEYS * (dimP + 8) * 2 + (size_t)DVB * 32 * VT_STRIDE * 2;
+  const size_t lds = ((size_t)TB_KEYS * (dimP + 8) * 2 + (size_t)DVB * 32 * VT_STRIDE * 2) *
+                     (PREFETCH ? 2 : 1);
   auto kern = window_attn_mfma_k<DKT_MAX, DVB, PREFETCH>;
   kern<<<dim3(nwork, nsplit), 256, lds, s>>>((const short*)q, (const short*)pool, work, cu,
                                              seq_start, table, maxb, bs, (bf16*)out, part, H, G,
